@@ -1,0 +1,713 @@
+// C-ABI of libhfuse_gfx950: configuration, plans, argument validation and the
+// host launcher.  Compiled as HIP host code; no kernels live in this file.
+#include <hip/hip_runtime.h>
+
+#include <algorithm>
+#include <cstring>
+#include <fstream>
+#include <mutex>
+#include <sstream>
+#include <string>
+#include <vector>
+
+#include "../../include/hfuse_gfx950.h"
+#include "device/crypto_bodies.h"
+#include "device/dl_bodies.h"
+#include "fusion_model.h"
+#include "launch.h"
+
+using namespace hfuse;
+
+// ---------------------------------------------------------------- error state
+namespace {
+
+thread_local std::string g_error;
+
+int fail(int code, const std::string &msg) {
+  g_error = msg;
+  return code;
+}
+
+int hip_fail(hipError_t e, const char *what) {
+  return fail(HF_EHIP, std::string(what) + ": " + hipGetErrorString(e));
+}
+
+struct KernelName {
+  const char *name;
+  KernelId id;
+};
+const KernelName kNames[] = {
+    {"im2col_kernel", K_IM2COL},
+    {"MaxPoolForward", K_MAXPOOL},
+    {"batch_norm_collect_statistics_kernel", K_BNSTATS},
+    {"upsample_nearest2d_out_frame", K_UPSAMPLE_NEAREST},
+    {"kernelHistogram1D", K_HISTC},
+    {"ethash_search", K_ETHASH},
+    // the reference clones ethash_search so each pair has its own symbol (configs/ethash_sha256.yaml:7)
+    {"ethash_search2", K_ETHASH},
+    {"ethash_search3", K_ETHASH},
+    {"ethash_search4", K_ETHASH},
+    {"sha256d_gpu_hash_shared", K_SHA256D},
+    {"sia_blake2b_gpu_hash", K_SIA_BLAKE2B},
+    {"blake2b_gpu_hash", K_BLAKE2B},
+};
+
+bool lookup_kernel(const std::string &name, KernelId &id) {
+  for (auto &k : kNames)
+    if (name == k.name) {
+      id = k.id;
+      return true;
+    }
+  return false;
+}
+
+// Barriers each built body executes (the YAML's HasBarriers is informational in the
+// reference as well: BarrierRewriter rewrites whatever __syncthreads it finds).
+bool body_has_barriers(KernelId id) { return id == K_BNSTATS || id == K_HISTC; }
+
+// ------------------------------------------------ constants of the searches
+struct SearchConstants {
+  std::mutex mu;
+  // ethash
+  const void *dag = nullptr;
+  uint32_t dag_items = 0;
+  uint64_t eth_header[4] = {0, 0, 0, 0};
+  uint64_t eth_target = 0;
+  bool eth_set = false;
+  // sha256d
+  uint32_t sha_mid[8];
+  uint32_t sha_tail[3];
+  uint64_t sha_target = 0;
+  bool sha_set = false;
+  // blake2b headers
+  uint64_t sia_m[10];
+  bool sia_set = false;
+  uint64_t b2_m[10];
+  bool b2_set = false;
+} g_const;
+
+uint32_t load_be32(const uint8_t *p) {
+  return ((uint32_t)p[0] << 24) | ((uint32_t)p[1] << 16) | ((uint32_t)p[2] << 8) | p[3];
+}
+uint64_t load_le64(const uint8_t *p) {
+  uint64_t v = 0;
+  for (int i = 7; i >= 0; i--) v = (v << 8) | p[i];
+  return v;
+}
+uint32_t rotr(uint32_t x, int n) { return (x >> n) | (x << (32 - n)); }
+
+// Host SHA-256 compression, used once per header for the midstate.
+void host_sha256_compress(uint32_t st[8], const uint32_t blk[16]) {
+  static const uint32_t K[64] = {
+      0x428a2f98, 0x71374491, 0xb5c0fbcf, 0xe9b5dba5, 0x3956c25b, 0x59f111f1, 0x923f82a4, 0xab1c5ed5,
+      0xd807aa98, 0x12835b01, 0x243185be, 0x550c7dc3, 0x72be5d74, 0x80deb1fe, 0x9bdc06a7, 0xc19bf174,
+      0xe49b69c1, 0xefbe4786, 0x0fc19dc6, 0x240ca1cc, 0x2de92c6f, 0x4a7484aa, 0x5cb0a9dc, 0x76f988da,
+      0x983e5152, 0xa831c66d, 0xb00327c8, 0xbf597fc7, 0xc6e00bf3, 0xd5a79147, 0x06ca6351, 0x14292967,
+      0x27b70a85, 0x2e1b2138, 0x4d2c6dfc, 0x53380d13, 0x650a7354, 0x766a0abb, 0x81c2c92e, 0x92722c85,
+      0xa2bfe8a1, 0xa81a664b, 0xc24b8b70, 0xc76c51a3, 0xd192e819, 0xd6990624, 0xf40e3585, 0x106aa070,
+      0x19a4c116, 0x1e376c08, 0x2748774c, 0x34b0bcb5, 0x391c0cb3, 0x4ed8aa4a, 0x5b9cca4f, 0x682e6ff3,
+      0x748f82ee, 0x78a5636f, 0x84c87814, 0x8cc70208, 0x90befffa, 0xa4506ceb, 0xbef9a3f7, 0xc67178f2};
+  uint32_t w[64];
+  for (int i = 0; i < 16; i++) w[i] = blk[i];
+  for (int i = 16; i < 64; i++)
+    w[i] = w[i - 16] + (rotr(w[i - 15], 7) ^ rotr(w[i - 15], 18) ^ (w[i - 15] >> 3)) + w[i - 7] +
+           (rotr(w[i - 2], 17) ^ rotr(w[i - 2], 19) ^ (w[i - 2] >> 10));
+  uint32_t v[8];
+  for (int i = 0; i < 8; i++) v[i] = st[i];
+  for (int i = 0; i < 64; i++) {
+    uint32_t t1 = v[7] + (rotr(v[4], 6) ^ rotr(v[4], 11) ^ rotr(v[4], 25)) + ((v[4] & v[5]) ^ (~v[4] & v[6])) + K[i] + w[i];
+    uint32_t t2 = (rotr(v[0], 2) ^ rotr(v[0], 13) ^ rotr(v[0], 22)) + ((v[0] & v[1]) ^ (v[0] & v[2]) ^ (v[1] & v[2]));
+    for (int j = 7; j > 0; j--) v[j] = v[j - 1];
+    v[4] += t1;
+    v[0] = t1 + t2;
+  }
+  for (int i = 0; i < 8; i++) st[i] += v[i];
+}
+
+// ------------------------------------------------------------ device facts
+int g_cu_count = 0;
+int cu_count() {
+  if (g_cu_count == 0) {
+    int dev = 0;
+    hipDeviceProp_t prop;
+    if (hipGetDevice(&dev) == hipSuccess && hipGetDeviceProperties(&prop, dev) == hipSuccess)
+      g_cu_count = prop.multiProcessorCount;
+    if (g_cu_count <= 0) g_cu_count = 256;
+  }
+  return g_cu_count;
+}
+
+// ------------------------------------------------------- argument validation
+struct Prepared {
+  KernelId id = K_COUNT;
+  alignas(16) unsigned char blob[320];  // device-side argument struct
+  unsigned hint = 0;
+  unsigned lds = 0;
+  bool exact_grid = false;  // the grid decides the amount of work (ethash)
+  unsigned long long items = 0;  // work items of one pass at the chosen hint
+};
+
+bool aligned16(const void *p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
+
+int prepare_im2col(const hf_im2col_args &a, Prepared &p) {
+  if (!a.data_im || !a.data_col) return fail(HF_EINVAL, "im2col_kernel: null data pointer");
+  if (a.n < 0 || a.height <= 0 || a.width <= 0 || a.kernel_h <= 0 || a.kernel_w <= 0 || a.stride_h <= 0 ||
+      a.stride_w <= 0 || a.dilation_h <= 0 || a.dilation_w <= 0 || a.height_col <= 0 || a.width_col <= 0 ||
+      a.pad_h < 0 || a.pad_w < 0)
+    return fail(HF_EINVAL, "im2col_kernel: non-positive geometry");
+  if (a.n % (a.height_col * a.width_col) != 0)
+    return fail(HF_EINVAL, "im2col_kernel: n is not channels * height_col * width_col");
+  const int64_t hc = (a.height + 2 * a.pad_h - (a.dilation_h * (a.kernel_h - 1) + 1)) / a.stride_h + 1;
+  const int64_t wc = (a.width + 2 * a.pad_w - (a.dilation_w * (a.kernel_w - 1) + 1)) / a.stride_w + 1;
+  if (hc != a.height_col || wc != a.width_col)
+    return fail(HF_EINVAL, "im2col_kernel: height_col/width_col do not follow from the geometry");
+  std::memcpy(p.blob, &a, sizeof a);
+  const int64_t channels = a.n / (a.height_col * a.width_col);
+  const bool fast = a.kernel_h == 3 && a.kernel_w == 3 && a.stride_h == 1 && a.stride_w == 1 && a.pad_h == 1 &&
+                    a.pad_w == 1 && a.dilation_h == 1 && a.dilation_w == 1 && a.width % 4 == 0 &&
+                    aligned16(a.data_im) && aligned16(a.data_col) &&
+                    channels * 9 * a.height * a.width < (int64_t)1 << 31;
+  p.hint = fast ? HINT_IM2COL_3X3_S1P1 : HINT_GENERIC;
+  p.items = fast ? (unsigned long long)a.n / 4 : (unsigned long long)a.n;
+  return HF_OK;
+}
+
+int prepare_maxpool(const hf_maxpool_args &a, Prepared &p) {
+  if (!a.bottom_data || !a.top_data || !a.top_mask) return fail(HF_EINVAL, "MaxPoolForward: null data pointer");
+  if (a.nthreads < 0 || a.num <= 0 || a.channels <= 0 || a.height <= 0 || a.width <= 0 || a.pooled_height <= 0 ||
+      a.pooled_width <= 0 || a.kernel_h <= 0 || a.kernel_w <= 0 || a.stride_h <= 0 || a.stride_w <= 0 ||
+      a.pad_h < 0 || a.pad_w < 0 || a.dilation_h <= 0 || a.dilation_w <= 0)
+    return fail(HF_EINVAL, "MaxPoolForward: non-positive geometry");
+  if ((int64_t)a.nthreads != (int64_t)a.num * a.channels * a.pooled_height * a.pooled_width)
+    return fail(HF_EINVAL, "MaxPoolForward: nthreads is not num * channels * pooled_height * pooled_width");
+  if (a.pad_h * 2 > (a.kernel_h - 1) * a.dilation_h + 1 || a.pad_w * 2 > (a.kernel_w - 1) * a.dilation_w + 1)
+    return fail(HF_EINVAL, "MaxPoolForward: pad should be at most half of the effective kernel size");
+  if ((a.pooled_height - 1) * a.stride_h - a.pad_h >= a.height || (a.pooled_width - 1) * a.stride_w - a.pad_w >= a.width)
+    return fail(HF_EINVAL, "MaxPoolForward: last window starts outside the input");
+  std::memcpy(p.blob, &a, sizeof a);
+  const bool common = a.stride_h == 2 && a.stride_w == 2 && a.dilation_h == 1 && a.dilation_w == 1 &&
+                      a.width % 8 == 0 && a.pooled_width * 2 == a.width && a.pooled_width % 4 == 0 &&
+                      aligned16(a.bottom_data) && aligned16(a.top_data) && aligned16(a.top_mask) &&
+                      (int64_t)a.num * a.channels * a.height * a.width < (int64_t)1 << 31;
+  p.hint = HINT_GENERIC;
+  if (common && a.kernel_h == 3 && a.kernel_w == 3 && a.pad_h == 1 && a.pad_w == 1 &&
+      a.pooled_height == (a.height + 2 - 3) / 2 + 1)
+    p.hint = HINT_POOL_K3S2P1;
+  if (common && a.kernel_h == 2 && a.kernel_w == 2 && a.pad_h == 0 && a.pad_w == 0 &&
+      a.pooled_height == (a.height - 2) / 2 + 1)
+    p.hint = HINT_POOL_K2S2P0;
+  p.items = p.hint ? (unsigned long long)a.nthreads / 4 : (unsigned long long)a.nthreads;
+  return HF_OK;
+}
+
+int prepare_bn(const hf_bn_stats_args &a, Prepared &p) {
+  if (!a.input.data || !a.save_mean.data || !a.save_transformed_var.data)
+    return fail(HF_EINVAL, "batch_norm_collect_statistics_kernel: null data pointer");
+  if (a.input.sizes[0] <= 0 || a.input.sizes[1] <= 0 || a.input.sizes[2] <= 0)
+    return fail(HF_EINVAL, "batch_norm_collect_statistics_kernel: empty input");
+  if (a.save_mean.sizes[0] != a.input.sizes[1] || a.save_transformed_var.sizes[0] != a.input.sizes[1])
+    return fail(HF_EINVAL, "batch_norm_collect_statistics_kernel: output length is not the channel count");
+  for (int i = 0; i < 3; i++)
+    if (a.input.strides[i] < 0) return fail(HF_EINVAL, "batch_norm_collect_statistics_kernel: negative stride");
+  std::memcpy(p.blob, &a, sizeof a);
+  const bool fast = a.input.strides[2] == 1 && a.input.sizes[2] % 4 == 0 && a.input.strides[0] % 4 == 0 &&
+                    a.input.strides[1] % 4 == 0 && aligned16(a.input.data);
+  p.hint = fast ? HINT_BN_VEC4 : HINT_GENERIC;
+  p.lds = BnStatsBody::kLdsBytes;
+  p.items = (unsigned long long)a.input.sizes[1];  // planes
+  return HF_OK;
+}
+
+int prepare_upsample(const hf_upsample_nearest_args &a, Prepared &p) {
+  if (!a.idata || !a.odata) return fail(HF_EINVAL, "upsample_nearest2d_out_frame: null data pointer");
+  if (a.nc == 0 || a.height1 == 0 || a.width1 == 0 || a.height2 == 0 || a.width2 == 0)
+    return fail(HF_EINVAL, "upsample_nearest2d_out_frame: empty tensor");
+  if (!(a.height_scale > 0.0f) || !(a.width_scale > 0.0f))
+    return fail(HF_EINVAL, "upsample_nearest2d_out_frame: scale must be positive");
+  std::memcpy(p.blob, &a, sizeof a);
+  const bool fast = a.height2 == 2 * a.height1 && a.width2 == 2 * a.width1 && a.height_scale == 0.5f &&
+                    a.width_scale == 0.5f && a.width1 % 4 == 0 && aligned16(a.idata) && aligned16(a.odata) &&
+                    a.nc * a.height2 * a.width2 < (size_t)1 << 32;
+  p.hint = fast ? HINT_UP_2X : HINT_GENERIC;
+  p.items = fast ? a.nc * a.height1 * (a.width1 / 4) : a.nc * a.height2 * a.width2;
+  return HF_OK;
+}
+
+int prepare_histc(const hf_histc_args &a, Prepared &p) {
+  if (!a.a.data || !a.b.data) return fail(HF_EINVAL, "kernelHistogram1D: null data pointer");
+  if (a.nbins <= 0) return fail(HF_EINVAL, "kernelHistogram1D: bins must be > 0");
+  if (!(a.minvalue < a.maxvalue)) return fail(HF_EINVAL, "kernelHistogram1D: max must be larger than min");
+  if (a.total_elements < 0) return fail(HF_EINVAL, "kernelHistogram1D: negative element count");
+  if (a.a.dims != 1 || a.b.dims != 1)
+    return fail(HF_EUNSUPPORTED, "kernelHistogram1D: only 1-D tensors are built");
+  if (a.a.sizes[0] != a.nbins) return fail(HF_EINVAL, "kernelHistogram1D: output length is not nbins");
+  if (a.b.sizes[0] != a.total_elements) return fail(HF_EINVAL, "kernelHistogram1D: totalElements is not the input length");
+  if (a.a.strides[0] != 1) return fail(HF_EUNSUPPORTED, "kernelHistogram1D: output must be contiguous");
+  if (a.nbins > 15360) return fail(HF_EUNSUPPORTED, "kernelHistogram1D: more bins than fit the LDS budget (15360)");
+  std::memcpy(p.blob, &a, sizeof a);
+  const bool fast = a.b.strides[0] == 1 && aligned16(a.b.data);
+  p.hint = fast ? HINT_HIST_VEC4 : HINT_GENERIC;
+  p.lds = (unsigned)a.nbins * 4u;
+  p.items = fast ? (unsigned long long)(a.total_elements + 3) / 4 : (unsigned long long)a.total_elements;
+  return HF_OK;
+}
+
+int prepare_ethash(const hf_ethash_args &a, Prepared &p) {
+  if (!a.g_output) return fail(HF_EINVAL, "ethash_search: null result pointer");
+  std::lock_guard<std::mutex> lock(g_const.mu);
+  if (!g_const.eth_set) return fail(HF_EINVAL, "ethash_search: hf_ethash_set_constants has not been called");
+  EthashDevArgs d;
+  d.out = a.g_output;
+  d.start_nonce = a.start_nonce;
+  d.dag = static_cast<const u32x4 *>(g_const.dag);
+  d.n_items = g_const.dag_items;
+  d.pow2_mask = (d.n_items & (d.n_items - 1)) == 0 ? d.n_items - 1 : 0;
+  d.target = g_const.eth_target;
+  std::memcpy(d.header, g_const.eth_header, sizeof d.header);
+  static_assert(sizeof(EthashDevArgs) <= sizeof(p.blob), "blob too small");
+  std::memcpy(p.blob, &d, sizeof d);
+  p.exact_grid = true;
+  return HF_OK;
+}
+
+int prepare_sha256d(const hf_sha256d_args &a, Prepared &p) {
+  if (!a.res_nonces) return fail(HF_EINVAL, "sha256d_gpu_hash_shared: null result pointer");
+  std::lock_guard<std::mutex> lock(g_const.mu);
+  if (!g_const.sha_set) return fail(HF_EINVAL, "sha256d_gpu_hash_shared: hf_sha256d_set_block has not been called");
+  Sha256dDevArgs d;
+  d.threads = a.threads;
+  d.start_nonce = a.start_nonce;
+  d.out = reinterpret_cast<hf_search_results *>(a.res_nonces);
+  std::memcpy(d.midstate, g_const.sha_mid, sizeof d.midstate);
+  std::memcpy(d.tail, g_const.sha_tail, sizeof d.tail);
+  d.pad = 0;
+  d.target64 = g_const.sha_target;
+  std::memcpy(p.blob, &d, sizeof d);
+  p.items = a.threads;
+  return HF_OK;
+}
+
+int prepare_blake2b(const hf_blake2b_args &a, bool sia, Prepared &p) {
+  const char *who = sia ? "sia_blake2b_gpu_hash" : "blake2b_gpu_hash";
+  if (!a.res_nonce) return fail(HF_EINVAL, std::string(who) + ": null result pointer");
+  std::lock_guard<std::mutex> lock(g_const.mu);
+  if (!(sia ? g_const.sia_set : g_const.b2_set))
+    return fail(HF_EINVAL, std::string(who) + ": the header block has not been set");
+  Blake2bDevArgs d;
+  d.threads = a.threads;
+  d.start_nonce = a.start_nonce;
+  d.out = reinterpret_cast<hf_search_results *>(a.res_nonce);
+  d.target64 = ((uint64_t)a.target2[1] << 32) | a.target2[0];
+  std::memcpy(d.m, sia ? g_const.sia_m : g_const.b2_m, sizeof d.m);
+  std::memcpy(p.blob, &d, sizeof d);
+  p.items = a.threads;
+  return HF_OK;
+}
+
+int prepare(KernelId id, const void *args, Prepared &p) {
+  if (!args) return fail(HF_EINVAL, "null argument list");
+  p = Prepared();
+  p.id = id;
+  switch (id) {
+    case K_IM2COL: return prepare_im2col(*static_cast<const hf_im2col_args *>(args), p);
+    case K_MAXPOOL: return prepare_maxpool(*static_cast<const hf_maxpool_args *>(args), p);
+    case K_BNSTATS: return prepare_bn(*static_cast<const hf_bn_stats_args *>(args), p);
+    case K_UPSAMPLE_NEAREST: return prepare_upsample(*static_cast<const hf_upsample_nearest_args *>(args), p);
+    case K_HISTC: return prepare_histc(*static_cast<const hf_histc_args *>(args), p);
+    case K_ETHASH: return prepare_ethash(*static_cast<const hf_ethash_args *>(args), p);
+    case K_SHA256D: return prepare_sha256d(*static_cast<const hf_sha256d_args *>(args), p);
+    case K_SIA_BLAKE2B: return prepare_blake2b(*static_cast<const hf_blake2b_args *>(args), true, p);
+    case K_BLAKE2B: return prepare_blake2b(*static_cast<const hf_blake2b_args *>(args), false, p);
+    default: return fail(HF_ENOTFOUND, "unknown kernel id");
+  }
+}
+
+// Blocks one pass of `p` wants when it owns `threads` threads per block.
+unsigned long long wanted_blocks(const Prepared &p, unsigned threads) {
+  if (p.id == K_BNSTATS) return p.items;
+  return (p.items + threads - 1) / threads;
+}
+
+// Default grid: enough resident workgroups to fill every CU twice over, never
+// more than the work asks for.  Streaming bodies stride over the rest.
+unsigned default_grid(unsigned long long want, unsigned block_threads) {
+  const unsigned per_cu = std::max(1u, 2048u / block_threads);
+  const unsigned long long cap = (unsigned long long)cu_count() * per_cu * 2ull;
+  unsigned long long g = std::min(std::max(want, 1ull), cap);
+  return (unsigned)g;
+}
+
+constexpr unsigned kDefaultEthashGrid = 8192;  // the authors' launches: scripts/data/ethminer_event.csv
+
+int do_launch_native(KernelId id, const Prepared &p, int grid_blocks, unsigned block, hipStream_t stream) {
+  if (block == 0 || block % kWave != 0 || block > (is_crypto(id) ? 512u : kMaxBlock))
+    return fail(HF_EINVAL, "block size must be a multiple of 64 within the kernel's launch bound");
+  unsigned grid;
+  if (grid_blocks > 0) grid = (unsigned)grid_blocks;
+  else if (p.exact_grid) grid = kDefaultEthashGrid;
+  else grid = default_grid(wanted_blocks(p, block), block);
+  if (!p.exact_grid && p.items == 0) return HF_OK;  // nothing to do
+  hipError_t e = is_crypto(id) ? launch_native_crypto(id, p.blob, p.hint, grid, block, p.lds, stream)
+                               : launch_native_dl(id, p.blob, p.hint, grid, block, p.lds, stream);
+  if (e != hipSuccess) return hip_fail(e, "native launch");
+  return HF_OK;
+}
+
+}  // namespace
+
+// ------------------------------------------------------------------ opaque types
+struct hf_config {
+  Config cfg;
+};
+
+struct hf_plan {
+  KernelRow rows[2];
+  KernelId ids[2];
+  const Preset *preset;
+  Partition part;
+  int barrier_mode;
+};
+
+// ------------------------------------------------------------------ C-ABI
+extern "C" {
+
+HF_API const char *hf_last_error(void) { return g_error.c_str(); }
+HF_API int hf_version(void) { return 100; }
+
+HF_API int hf_config_load_text(const char *fusion_yaml, const char *kernels_yaml, hf_config **out) {
+  if (!out) return fail(HF_EINVAL, "null output pointer");
+  *out = nullptr;
+  if (!kernels_yaml) return fail(HF_EINVAL, "null kernel table");
+  auto *c = new hf_config();
+  std::string err;
+  if (!parse_config(fusion_yaml, kernels_yaml, c->cfg, err)) {
+    delete c;
+    return fail(HF_EPARSE, err);
+  }
+  *out = c;
+  return HF_OK;
+}
+
+HF_API int hf_config_load_files(const char *fusion_path, const char *kernels_path, hf_config **out) {
+  if (!out) return fail(HF_EINVAL, "null output pointer");
+  *out = nullptr;
+  if (!kernels_path) return fail(HF_EINVAL, "null kernel table path");
+  auto slurp = [](const char *path, std::string &dst) {
+    std::ifstream in(path, std::ios::binary);
+    if (!in) return false;
+    std::ostringstream ss;
+    ss << in.rdbuf();
+    dst = ss.str();
+    return true;
+  };
+  std::string f, k;
+  if (!slurp(kernels_path, k)) return fail(HF_EIO, std::string("failed to read configs: ") + kernels_path);
+  if (fusion_path && !slurp(fusion_path, f)) return fail(HF_EIO, std::string("failed to read configs: ") + fusion_path);
+  return hf_config_load_text(fusion_path ? f.c_str() : nullptr, k.c_str(), out);
+}
+
+HF_API void hf_config_free(hf_config *cfg) { delete cfg; }
+
+HF_API int hf_config_num_fusions(const hf_config *cfg) { return cfg ? (int)cfg->cfg.fusions.size() : fail(HF_EINVAL, "null config"); }
+HF_API int hf_config_num_kernels(const hf_config *cfg) { return cfg ? (int)cfg->cfg.rows.size() : fail(HF_EINVAL, "null config"); }
+
+HF_API int hf_config_fusion(const hf_config *cfg, int i, const char **file, const char **k1, const char **k2) {
+  if (!cfg) return fail(HF_EINVAL, "null config");
+  if (i < 0 || i >= (int)cfg->cfg.fusions.size()) return fail(HF_EINVAL, "fusion index out of range");
+  const FusionRow &f = cfg->cfg.fusions[i];
+  if (file) *file = f.file.c_str();
+  if (k1) *k1 = f.kernels[0].c_str();
+  if (k2) *k2 = f.kernels[1].c_str();
+  return HF_OK;
+}
+
+HF_API int hf_config_kernel(const hf_config *cfg, const char *name, hf_kernel_info *out) {
+  if (!cfg || !name || !out) return fail(HF_EINVAL, "null argument");
+  const KernelRow *r = cfg->cfg.find(name);
+  if (!r) return fail(HF_ENOTFOUND, std::string("kernel '") + name + "' is not in the kernel table");
+  std::memset(out, 0, sizeof *out);
+  std::strncpy(out->kernel_name, r->name.c_str(), sizeof out->kernel_name - 1);
+  out->has_barriers = r->has_barriers;
+  out->block_dim = {r->block_dim.x, r->block_dim.y, r->block_dim.z};
+  out->reg = r->reg;
+  out->exec_time = r->exec_time;
+  return HF_OK;
+}
+
+HF_API int hf_plan_num_splits(const hf_config *cfg, int fusion_index) {
+  if (!cfg) return fail(HF_EINVAL, "null config");
+  if (fusion_index < 0 || fusion_index >= (int)cfg->cfg.fusions.size()) return fail(HF_EINVAL, "fusion index out of range");
+  const FusionRow &f = cfg->cfg.fusions[fusion_index];
+  return num_splits(*cfg->cfg.find(f.kernels[0]), *cfg->cfg.find(f.kernels[1]));
+}
+
+HF_API int hf_plan_create(const hf_config *cfg, int fusion_index, const char *preset, int split_idx, int split_threads,
+                          hf_plan **out) {
+  if (!out) return fail(HF_EINVAL, "null output pointer");
+  *out = nullptr;
+  if (!cfg || !preset) return fail(HF_EINVAL, "null argument");
+  if (fusion_index < 0 || fusion_index >= (int)cfg->cfg.fusions.size()) return fail(HF_EINVAL, "fusion index out of range");
+  const Preset *p = find_preset(preset);
+  if (!p) return fail(HF_ENOTFOUND, std::string("unknown preset '") + preset + "' (vfuse_lb, vfuse, hfuse, hfuse_lb)");
+  if (split_threads > 0 && split_threads % (int)kWave != 0)
+    return fail(HF_EINVAL, "split_threads must be a multiple of the 64-lane wavefront");
+  const FusionRow &f = cfg->cfg.fusions[fusion_index];
+  auto plan = new hf_plan();
+  plan->preset = p;
+  for (int i = 0; i < 2; i++) {
+    plan->rows[i] = *cfg->cfg.find(f.kernels[i]);
+    if (!lookup_kernel(plan->rows[i].name, plan->ids[i])) {
+      int code = plan->rows[i].name == "upsample_bilinear2d_out_frame" ? HF_EUNSUPPORTED : HF_ENOTFOUND;
+      std::string msg = "kernel '" + plan->rows[i].name + "' has no gfx950 implementation in this library";
+      delete plan;
+      return fail(code, msg);
+    }
+  }
+  if (is_crypto(plan->ids[0]) != is_crypto(plan->ids[1])) {
+    delete plan;
+    return fail(HF_EUNSUPPORTED, "pairs mixing a tensor kernel with a search kernel are not built");
+  }
+  std::string err;
+  int rc = make_partition(plan->rows[0], plan->rows[1], *p, split_idx, split_threads, plan->part, err);
+  if (rc != HF_OK) {
+    delete plan;
+    return fail(rc, err);
+  }
+  if (is_crypto(plan->ids[0]) && !p->base_line && plan->part.launch_threads > 512) {
+    delete plan;
+    return fail(HF_EINVAL, "search kernels are built for fused blocks of at most 512 threads");
+  }
+  const bool b1 = body_has_barriers(plan->ids[0]), b2 = body_has_barriers(plan->ids[1]);
+  // One barrier policy per pair: nothing to do when neither body synchronises;
+  // an LDS-counter barrier scoped to the synchronising half otherwise.  (Both
+  // tensor bodies that synchronise do so twice per block, so a pair of them may
+  // also share the hardware barrier: HF_BARRIER_MATCHED via hf_plan_set_barrier_mode.)
+  plan->barrier_mode = (b1 || b2) ? HF_BARRIER_SUBSET : HF_BARRIER_NONE;
+  *out = plan;
+  return HF_OK;
+}
+
+HF_API int hf_plan_set_barrier_mode(hf_plan *plan, int mode) {
+  if (!plan) return fail(HF_EINVAL, "null plan");
+  const bool b1 = body_has_barriers(plan->ids[0]), b2 = body_has_barriers(plan->ids[1]);
+  switch (mode) {
+    case HF_BARRIER_NONE:
+      if (b1 || b2) return fail(HF_EINVAL, "this pair synchronises; HF_BARRIER_NONE is not legal");
+      break;
+    case HF_BARRIER_SUBSET:
+      if (!b1 && !b2) return fail(HF_EINVAL, "neither kernel synchronises; nothing to scope");
+      break;
+    case HF_BARRIER_MATCHED:
+      if (!(b1 && b2)) return fail(HF_EINVAL, "matched s_barrier needs both halves to synchronise equally often");
+      break;
+    case HF_BARRIER_BLOCKIDX:
+      break;
+    default:
+      return fail(HF_EINVAL, "unknown barrier mode");
+  }
+  plan->barrier_mode = mode;
+  return HF_OK;
+}
+
+HF_API void hf_plan_free(hf_plan *plan) { delete plan; }
+
+HF_API int hf_plan_partition(const hf_plan *plan, hf_partition *out) {
+  if (!plan || !out) return fail(HF_EINVAL, "null argument");
+  std::memset(out, 0, sizeof *out);
+  std::strncpy(out->name, plan->part.name.c_str(), sizeof out->name - 1);
+  for (int i = 0; i < 2; i++) {
+    out->lo[i] = plan->part.lo[i];
+    out->hi[i] = plan->part.hi[i];
+    out->block_dim[i] = {plan->part.block_dim[i].x, plan->part.block_dim[i].y, plan->part.block_dim[i].z};
+  }
+  out->launch_threads = plan->part.launch_threads;
+  out->launch_blocks = plan->part.launch_blocks;
+  out->barrier_mode = plan->barrier_mode;
+  return HF_OK;
+}
+
+HF_API int hf_plan_local_index(const hf_plan *plan, int half, uint32_t tid, hf_dim3 *out) {
+  if (!plan || !out) return fail(HF_EINVAL, "null argument");
+  if (half < 0 || half > 1) return fail(HF_EINVAL, "half must be 0 or 1");
+  if (tid < plan->part.lo[half] || tid >= plan->part.hi[half])
+    return fail(HF_EINVAL, "thread is outside this kernel's bounds");
+  Dim3 d = local_index(tid, plan->part.lo[half], plan->part.block_dim[half]);
+  *out = {d.x, d.y, d.z};
+  return HF_OK;
+}
+
+// ------------------------------------------------------------- constants
+HF_API int hf_ethash_set_constants(const void *dag, uint32_t dag_items, const uint8_t header[32], uint64_t target,
+                                   void *) {
+  if (!dag || !header) return fail(HF_EINVAL, "ethash: null dag or header");
+  if (dag_items == 0) return fail(HF_EINVAL, "ethash: empty dag");
+  if (!aligned16(dag)) return fail(HF_EINVAL, "ethash: dag must be 16-byte aligned");
+  std::lock_guard<std::mutex> lock(g_const.mu);
+  g_const.dag = dag;
+  g_const.dag_items = dag_items;
+  for (int i = 0; i < 4; i++) g_const.eth_header[i] = load_le64(header + 8 * i);
+  g_const.eth_target = target;
+  g_const.eth_set = true;
+  return HF_OK;
+}
+
+HF_API int hf_sha256d_set_block(const uint8_t header[80], uint64_t target64, void *) {
+  if (!header) return fail(HF_EINVAL, "sha256d: null header");
+  uint32_t st[8] = {0x6a09e667, 0xbb67ae85, 0x3c6ef372, 0xa54ff53a, 0x510e527f, 0x9b05688c, 0x1f83d9ab, 0x5be0cd19};
+  uint32_t blk[16];
+  for (int i = 0; i < 16; i++) blk[i] = load_be32(header + 4 * i);
+  host_sha256_compress(st, blk);
+  std::lock_guard<std::mutex> lock(g_const.mu);
+  std::memcpy(g_const.sha_mid, st, sizeof st);
+  for (int i = 0; i < 3; i++) g_const.sha_tail[i] = load_be32(header + 64 + 4 * i);
+  g_const.sha_target = target64;
+  g_const.sha_set = true;
+  return HF_OK;
+}
+
+HF_API int hf_sia_blake2b_set_block(const uint8_t header[80], void *) {
+  if (!header) return fail(HF_EINVAL, "sia_blake2b: null header");
+  std::lock_guard<std::mutex> lock(g_const.mu);
+  for (int i = 0; i < 10; i++) g_const.sia_m[i] = load_le64(header + 8 * i);
+  g_const.sia_set = true;
+  return HF_OK;
+}
+
+HF_API int hf_blake2b_set_block(const uint8_t header[80], void *) {
+  if (!header) return fail(HF_EINVAL, "blake2b: null header");
+  std::lock_guard<std::mutex> lock(g_const.mu);
+  for (int i = 0; i < 10; i++) g_const.b2_m[i] = load_le64(header + 8 * i);
+  g_const.b2_set = true;
+  return HF_OK;
+}
+
+// ---------------------------------------------------------------- launches
+HF_API int hf_launch_native(const char *kernel_name, const void *args, int grid_blocks, int block_threads,
+                            void *stream) {
+  if (!kernel_name) return fail(HF_EINVAL, "null kernel name");
+  KernelId id;
+  if (!lookup_kernel(kernel_name, id))
+    return fail(HF_ENOTFOUND, std::string("kernel '") + kernel_name + "' has no gfx950 implementation in this library");
+  Prepared p;
+  int rc = prepare(id, args, p);
+  if (rc != HF_OK) return rc;
+  unsigned block = block_threads > 0 ? (unsigned)block_threads : (is_crypto(id) ? 128u : (id == K_MAXPOOL ? 256u : 512u));
+  return do_launch_native(id, p, grid_blocks, block, static_cast<hipStream_t>(stream));
+}
+
+namespace {
+
+int do_launch_fused(const hf_plan *plan, const Prepared &p1, const Prepared &p2, int grid_blocks, hipStream_t stream) {
+  if (plan->preset->base_line)
+    return fail(HF_EUNSUPPORTED, "vertical presets only report their partition; launch an hfuse preset");
+  FuseGeom g;
+  g.d1 = plan->part.hi[0] - plan->part.lo[0];
+  g.d2 = plan->part.hi[1] - plan->part.lo[1];
+  g.lds1 = (p1.lds + 15u) & ~15u;
+  g.lds2 = (p2.lds + 15u) & ~15u;
+  g.hint1 = p1.hint;
+  g.hint2 = p2.hint;
+  g.grid1 = g.grid2 = 0;
+  const bool crypto = is_crypto(plan->ids[0]);
+  const unsigned long long w1 = p1.exact_grid ? 0 : wanted_blocks(p1, g.d1);
+  const unsigned long long w2 = p2.exact_grid ? 0 : wanted_blocks(p2, g.d2);
+  hipError_t e;
+  if (plan->barrier_mode == HF_BARRIER_BLOCKIDX) {
+    // Each kernel gets its own workgroups inside one launch.
+    const unsigned block = std::max(g.d1, g.d2);
+    g.grid1 = p1.exact_grid ? (grid_blocks > 0 ? (unsigned)grid_blocks : kDefaultEthashGrid) : default_grid(w1, block);
+    g.grid2 = p2.exact_grid ? (grid_blocks > 0 ? (unsigned)grid_blocks : kDefaultEthashGrid) : default_grid(w2, block);
+    if (!p1.exact_grid && !p2.exact_grid && grid_blocks > 0) {
+      g.grid1 = std::max(1u, (unsigned)grid_blocks / 2);
+      g.grid2 = std::max(1u, (unsigned)grid_blocks - g.grid1);
+    }
+    const size_t lds = std::max(g.lds1, g.lds2);
+    e = crypto ? launch_fused_crypto(plan->ids[0], plan->ids[1], MODE_BLOCKIDX, p1.blob, p2.blob, g, g.grid1 + g.grid2, lds, stream)
+               : launch_fused_dl(plan->ids[0], plan->ids[1], MODE_BLOCKIDX, p1.blob, p2.blob, g, g.grid1 + g.grid2, lds, stream);
+  } else {
+    unsigned grid;
+    if (grid_blocks > 0) grid = (unsigned)grid_blocks;
+    else if (p1.exact_grid || p2.exact_grid) grid = kDefaultEthashGrid;
+    else grid = default_grid(std::max(w1, w2), g.d1 + g.d2);
+    const size_t lds = 4 * kBarrierWords + g.lds1 + g.lds2;
+    const FuseMode mode = plan->barrier_mode == HF_BARRIER_MATCHED ? MODE_MATCHED : MODE_HFUSE;
+    e = crypto ? launch_fused_crypto(plan->ids[0], plan->ids[1], mode, p1.blob, p2.blob, g, grid, lds, stream)
+               : launch_fused_dl(plan->ids[0], plan->ids[1], mode, p1.blob, p2.blob, g, grid, lds, stream);
+  }
+  if (e == hipErrorNotSupported) return fail(HF_EUNSUPPORTED, "this pair / barrier mode is not built");
+  if (e != hipSuccess) return hip_fail(e, "fused launch");
+  return HF_OK;
+}
+
+}  // namespace
+
+HF_API int hf_launch_fused(const hf_plan *plan, const void *args1, const void *args2, int grid_blocks, void *stream) {
+  if (!plan) return fail(HF_EINVAL, "null plan");
+  Prepared p1, p2;
+  int rc = prepare(plan->ids[0], args1, p1);
+  if (rc != HF_OK) return rc;
+  rc = prepare(plan->ids[1], args2, p2);
+  if (rc != HF_OK) return rc;
+  return do_launch_fused(plan, p1, p2, grid_blocks, static_cast<hipStream_t>(stream));
+}
+
+HF_API int hf_time_pair(const hf_plan *plan, int mode, const void *const *args1, const void *const *args2, int nsets,
+                        int warmup, int iters, int grid_blocks, void *stream_, float *elapsed_ms) {
+  if (!plan || !args1 || !args2 || !elapsed_ms) return fail(HF_EINVAL, "null argument");
+  if (nsets <= 0 || iters <= 0 || warmup < 0 || mode < 0 || mode > 3) return fail(HF_EINVAL, "bad repetition arguments");
+  hipStream_t stream = static_cast<hipStream_t>(stream_);
+  std::vector<Prepared> p1(nsets), p2(nsets);
+  for (int i = 0; i < nsets; i++) {
+    int rc = prepare(plan->ids[0], args1[i], p1[i]);
+    if (rc != HF_OK) return rc;
+    rc = prepare(plan->ids[1], args2[i], p2[i]);
+    if (rc != HF_OK) return rc;
+  }
+  const unsigned b1 = plan->rows[0].block_dim.size(), b2 = plan->rows[1].block_dim.size();
+  auto once = [&](int i) -> int {
+    const int s = i % nsets;
+    int rc = HF_OK;
+    if (mode == 0 || mode == 2) rc = do_launch_native(plan->ids[0], p1[s], mode == 2 ? 0 : grid_blocks, b1, stream);
+    if (rc != HF_OK) return rc;
+    if (mode == 1 || mode == 2) rc = do_launch_native(plan->ids[1], p2[s], mode == 2 ? 0 : grid_blocks, b2, stream);
+    if (rc != HF_OK) return rc;
+    if (mode == 3) rc = do_launch_fused(plan, p1[s], p2[s], grid_blocks, stream);
+    return rc;
+  };
+  for (int i = 0; i < warmup; i++) {
+    int rc = once(i);
+    if (rc != HF_OK) return rc;
+  }
+  hipEvent_t t0, t1;
+  hipError_t e = hipEventCreate(&t0);
+  if (e != hipSuccess) return hip_fail(e, "hipEventCreate");
+  e = hipEventCreate(&t1);
+  if (e != hipSuccess) { (void)hipEventDestroy(t0); return hip_fail(e, "hipEventCreate"); }
+  int rc = HF_OK;
+  e = hipEventRecord(t0, stream);
+  for (int i = 0; i < iters && rc == HF_OK && e == hipSuccess; i++) rc = once(warmup + i);
+  if (e == hipSuccess) e = hipEventRecord(t1, stream);
+  if (e == hipSuccess) e = hipEventSynchronize(t1);
+  if (e == hipSuccess) e = hipEventElapsedTime(elapsed_ms, t0, t1);
+  (void)hipEventDestroy(t0);
+  (void)hipEventDestroy(t1);
+  if (rc != HF_OK) return rc;
+  if (e != hipSuccess) return hip_fail(e, "timing");
+  return HF_OK;
+}
+
+HF_API int hf_fill_splitmix64(uint64_t *dst, uint64_t nwords, uint64_t seed, void *stream) {
+  if (!dst && nwords) return fail(HF_EINVAL, "null destination");
+  hipError_t e = launch_fill_splitmix64(reinterpret_cast<unsigned long long *>(dst), nwords, seed, static_cast<hipStream_t>(stream));
+  if (e != hipSuccess) return hip_fail(e, "fill launch");
+  return HF_OK;
+}
+
+HF_API int hf_copy_f32(const float *src, float *dst, uint64_t n, void *stream) {
+  if ((!src || !dst) && n) return fail(HF_EINVAL, "null pointer");
+  hipError_t e = launch_copy_f32(src, dst, n, static_cast<hipStream_t>(stream));
+  if (e != hipSuccess) return hip_fail(e, "copy launch");
+  return HF_OK;
+}
+
+}  // extern "C"

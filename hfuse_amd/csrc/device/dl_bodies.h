@@ -1,0 +1,413 @@
+// Device bodies of the five tensor kernels.  Each body is written once against
+// SubBlock and is instantiated both as a native kernel and as one half of a
+// fused kernel.  Every body has a general path that follows the original
+// kernel's semantics for any argument list, and a vectorised path (selected by
+// a host-validated hint) for the layouts that matter: 16-byte aligned rows,
+// stride-1 3x3 im2col, stride-2 pooling, exact 2x nearest upsampling.
+#pragma once
+#include <hip/hip_runtime.h>
+
+#include "../../../include/hfuse_gfx950.h"
+#include "subblock.h"
+
+namespace hfuse {
+
+// Hints (0 always means the general path).
+enum { HINT_GENERIC = 0, HINT_IM2COL_3X3_S1P1 = 1, HINT_POOL_K3S2P1 = 1, HINT_POOL_K2S2P0 = 2, HINT_UP_2X = 1, HINT_BN_VEC4 = 1, HINT_HIST_VEC4 = 1 };
+
+__device__ __forceinline__ f32x4 ld4(const float *p) { return *reinterpret_cast<const f32x4 *>(p); }
+__device__ __forceinline__ void st4(float *p, f32x4 v) { __builtin_nontemporal_store(v, reinterpret_cast<f32x4 *>(p)); }
+
+// ----------------------------------------------------------------------------
+// im2col_kernel<float>  (argument list: scripts/data/ml-event.csv:17)
+// One work item per (channel_in, h_out, w_out): kernel_h*kernel_w taps go to
+// rows channel_in*kh*kw + i*kw + j of the column matrix, zero outside the image.
+// ----------------------------------------------------------------------------
+struct Im2colBody {
+  using Args = hf_im2col_args;
+  static constexpr bool kBarriers = false;
+
+  template <class SB>
+  static __device__ void run(const Args &a, SB &sb, unsigned char *, unsigned hint) {
+    if (hint == HINT_IM2COL_3X3_S1P1) {
+      vec4_3x3(a, sb);
+      return;
+    }
+    const int64_t stride = (int64_t)sb.nblocks * sb.nthreads;
+    const int64_t plane_col = a.height_col * a.width_col;
+    for (int64_t index = (int64_t)sb.bid * sb.nthreads + sb.tid; index < a.n; index += stride) {
+      const int64_t w_out = index % a.width_col;
+      const int64_t idx = index / a.width_col;
+      const int64_t h_out = idx % a.height_col;
+      const int64_t channel_in = idx / a.height_col;
+      const int64_t channel_out = channel_in * a.kernel_h * a.kernel_w;
+      const int64_t h_in = h_out * a.stride_h - a.pad_h;
+      const int64_t w_in = w_out * a.stride_w - a.pad_w;
+      float *col = a.data_col + (channel_out * a.height_col + h_out) * a.width_col + w_out;
+      const float *im = a.data_im + (channel_in * a.height + h_in) * a.width + w_in;
+      for (int64_t i = 0; i < a.kernel_h; ++i) {
+        for (int64_t j = 0; j < a.kernel_w; ++j) {
+          const int64_t h = h_in + i * a.dilation_h, w = w_in + j * a.dilation_w;
+          *col = (h >= 0 && w >= 0 && h < a.height && w < a.width)
+                     ? im[i * a.dilation_h * a.width + j * a.dilation_w]
+                     : 0.0f;
+          col += plane_col;
+        }
+      }
+    }
+  }
+
+  // 3x3, stride 1, pad 1, dilation 1, width % 4 == 0: a work item owns four
+  // neighbouring output columns.  Per input row it needs columns w0-1 .. w0+4:
+  // one aligned 16-byte load plus the two edge scalars; each of the nine taps
+  // is then one 16-byte store.
+  template <class SB>
+  static __device__ __forceinline__ void vec4_3x3(const Args &a, SB &sb) {
+    const unsigned W = (unsigned)a.width, H = (unsigned)a.height;
+    const unsigned wq = W >> 2;
+    const unsigned plane = H * W;
+    const unsigned n4 = (unsigned)(a.n >> 2);
+    const unsigned stride = sb.nblocks * sb.nthreads;
+    for (unsigned idx4 = sb.bid * sb.nthreads + sb.tid; idx4 < n4; idx4 += stride) {
+      const unsigned w4 = idx4 % wq;
+      const unsigned t = idx4 / wq;
+      const unsigned h_out = t % H;
+      const unsigned c = t / H;
+      const unsigned w0 = w4 << 2;
+      const float *im = a.data_im + (size_t)c * plane;
+      float *col = a.data_col + (size_t)c * 9u * plane + (size_t)h_out * W + w0;
+      float r[3][6];
+#pragma unroll
+      for (int i = 0; i < 3; i++) {
+        const int h = (int)h_out - 1 + i;
+        if (h >= 0 && h < (int)H) {
+          const float *row = im + (unsigned)h * W + w0;
+          const f32x4 m = ld4(row);
+          r[i][0] = w0 > 0 ? row[-1] : 0.0f;
+          r[i][1] = m.x; r[i][2] = m.y; r[i][3] = m.z; r[i][4] = m.w;
+          r[i][5] = (w0 + 4 < W) ? row[4] : 0.0f;
+        } else {
+#pragma unroll
+          for (int k = 0; k < 6; k++) r[i][k] = 0.0f;
+        }
+      }
+#pragma unroll
+      for (int i = 0; i < 3; i++)
+#pragma unroll
+        for (int j = 0; j < 3; j++) {
+          f32x4 v = {r[i][j], r[i][j + 1], r[i][j + 2], r[i][j + 3]};
+          st4(col + (size_t)(i * 3 + j) * plane, v);
+        }
+    }
+  }
+};
+
+// ----------------------------------------------------------------------------
+// MaxPoolForward<float,float>  (argument list: scripts/data/ml-event.csv:5)
+// One work item per output; the window is scanned in (h, w) order and replaced
+// on `v > max || isnan(v)`, so ties keep the first index; the mask is h*W+w.
+// ----------------------------------------------------------------------------
+struct MaxPoolBody {
+  using Args = hf_maxpool_args;
+  static constexpr bool kBarriers = false;
+
+  template <class SB>
+  static __device__ void run(const Args &a, SB &sb, unsigned char *, unsigned hint) {
+    if (hint == HINT_POOL_K3S2P1) { vec4_s2<3, 1>(a, sb); return; }
+    if (hint == HINT_POOL_K2S2P0) { vec4_s2<2, 0>(a, sb); return; }
+    const int64_t stride = (int64_t)sb.nblocks * sb.nthreads;
+    for (int64_t index = (int64_t)sb.bid * sb.nthreads + sb.tid; index < a.nthreads; index += stride) {
+      const int pw = (int)(index % a.pooled_width);
+      const int ph = (int)((index / a.pooled_width) % a.pooled_height);
+      const int c = (int)((index / a.pooled_width / a.pooled_height) % a.channels);
+      const int n = (int)(index / a.pooled_width / a.pooled_height / a.channels);
+      int hstart = ph * a.stride_h - a.pad_h;
+      int wstart = pw * a.stride_w - a.pad_w;
+      const int hend = min(hstart + (a.kernel_h - 1) * a.dilation_h + 1, a.height);
+      const int wend = min(wstart + (a.kernel_w - 1) * a.dilation_w + 1, a.width);
+      while (hstart < 0) hstart += a.dilation_h;
+      while (wstart < 0) wstart += a.dilation_w;
+      float maxval = -INFINITY;
+      int maxidx = hstart * a.width + wstart;
+      const float *plane = a.bottom_data + ((int64_t)n * a.channels + c) * a.height * a.width;
+      for (int h = hstart; h < hend; h += a.dilation_h)
+        for (int w = wstart; w < wend; w += a.dilation_w) {
+          const float v = plane[h * a.width + w];
+          if ((v > maxval) || isnan(v)) {
+            maxidx = h * a.width + w;
+            maxval = v;
+          }
+        }
+      a.top_data[index] = maxval;
+      a.top_mask[index] = maxidx;
+    }
+  }
+
+  // K x K window, stride 2, pad P (K=3,P=1 or K=2,P=0), width % 8 == 0 and
+  // pooled_width == width/2: a work item owns four neighbouring outputs and
+  // reads, per window row, two aligned 16-byte vectors (+ the left edge for P=1).
+  template <int K, int P, class SB>
+  static __device__ __forceinline__ void vec4_s2(const Args &a, SB &sb) {
+    const unsigned W = (unsigned)a.width, H = (unsigned)a.height;
+    const unsigned PW = (unsigned)a.pooled_width, PH = (unsigned)a.pooled_height;
+    const unsigned pq = PW >> 2;
+    const unsigned n4 = (unsigned)a.nthreads >> 2;
+    const unsigned stride = sb.nblocks * sb.nthreads;
+    for (unsigned idx4 = sb.bid * sb.nthreads + sb.tid; idx4 < n4; idx4 += stride) {
+      const unsigned pw4 = idx4 % pq;
+      const unsigned t = idx4 / pq;
+      const unsigned ph = t % PH;
+      const unsigned nc = t / PH;
+      const float *plane = a.bottom_data + (size_t)nc * H * W;
+      const int hstart = (int)ph * 2 - P;
+      const unsigned wbase = pw4 << 3;
+      float maxv[4];
+      int maxi[4];
+      const int h0 = hstart < 0 ? 0 : hstart;
+#pragma unroll
+      for (int o = 0; o < 4; o++) {
+        const int ws = (int)wbase + 2 * o - P;
+        maxv[o] = -INFINITY;
+        maxi[o] = h0 * (int)W + (ws < 0 ? 0 : ws);
+      }
+#pragma unroll
+      for (int i = 0; i < K; i++) {
+        const int h = hstart + i;
+        if (h < 0 || h >= (int)H) continue;
+        const float *row = plane + (unsigned)h * W + wbase;
+        const f32x4 v0 = ld4(row), v1 = ld4(row + 4);
+        float vals[9];
+        // vals[k] is input column wbase - P + k
+        if (P == 1) {
+          vals[0] = wbase > 0 ? row[-1] : 0.0f;
+          vals[1] = v0.x; vals[2] = v0.y; vals[3] = v0.z; vals[4] = v0.w;
+          vals[5] = v1.x; vals[6] = v1.y; vals[7] = v1.z; vals[8] = v1.w;
+        } else {
+          vals[0] = v0.x; vals[1] = v0.y; vals[2] = v0.z; vals[3] = v0.w;
+          vals[4] = v1.x; vals[5] = v1.y; vals[6] = v1.z; vals[7] = v1.w;
+          vals[8] = 0.0f;
+        }
+        const int base_idx = h * (int)W + (int)wbase - P;
+#pragma unroll
+        for (int o = 0; o < 4; o++)
+#pragma unroll
+          for (int j = 0; j < K; j++) {
+            const int k = 2 * o + j;
+            if (P == 1 && k == 0 && wbase == 0) continue;  // column -1 is padding
+            const float v = vals[k];
+            if ((v > maxv[o]) || isnan(v)) {
+              maxv[o] = v;
+              maxi[o] = base_idx + k;
+            }
+          }
+      }
+      f32x4 ov = {maxv[0], maxv[1], maxv[2], maxv[3]};
+      st4(a.top_data + (size_t)idx4 * 4, ov);
+      i64x2 *mp = reinterpret_cast<i64x2 *>(a.top_mask + (size_t)idx4 * 4);
+      i64x2 m0 = {maxi[0], maxi[1]}, m1 = {maxi[2], maxi[3]};
+      __builtin_nontemporal_store(m0, mp);
+      __builtin_nontemporal_store(m1, mp + 1);
+    }
+  }
+};
+
+// ----------------------------------------------------------------------------
+// upsample_nearest2d_out_frame<float>: src = min((int)floorf(dst * scale), in - 1)
+// ----------------------------------------------------------------------------
+struct UpsampleNearestBody {
+  using Args = hf_upsample_nearest_args;
+  static constexpr bool kBarriers = false;
+
+  template <class SB>
+  static __device__ void run(const Args &a, SB &sb, unsigned char *, unsigned hint) {
+    if (hint == HINT_UP_2X) {
+      // Exact 2x: one 16-byte load feeds two output rows of two 16-byte stores each.
+      const unsigned w1q = (unsigned)a.width1 >> 2;
+      const unsigned h1 = (unsigned)a.height1;
+      const unsigned w2 = (unsigned)a.width2;
+      const unsigned n4 = (unsigned)(a.nc * a.height1) * w1q;
+      const unsigned stride = sb.nblocks * sb.nthreads;
+      for (unsigned idx = sb.bid * sb.nthreads + sb.tid; idx < n4; idx += stride) {
+        const unsigned x4 = idx % w1q;
+        const unsigned row = idx / w1q;  // c * h1 + y1
+        const f32x4 v = ld4(a.idata + (size_t)idx * 4);
+        // output row index: c*h2 + 2*y1 = 2*(c*h1 + y1)
+        float *o = a.odata + (size_t)row * 2u * w2 + (size_t)x4 * 8u;
+        const f32x4 lo = {v.x, v.x, v.y, v.y}, hi = {v.z, v.z, v.w, v.w};
+        st4(o, lo); st4(o + 4, hi);
+        st4(o + w2, lo); st4(o + w2 + 4, hi);
+        (void)h1;
+      }
+      return;
+    }
+    const size_t total = a.nc * a.height2 * a.width2;
+    const size_t stride = (size_t)sb.nblocks * sb.nthreads;
+    for (size_t index = (size_t)sb.bid * sb.nthreads + sb.tid; index < total; index += stride) {
+      const size_t x2 = index % a.width2;
+      const size_t y2 = (index / a.width2) % a.height2;
+      const size_t c = index / a.width2 / a.height2;
+      const int y1 = min((int)floorf((float)y2 * a.height_scale), (int)a.height1 - 1);
+      const int x1 = min((int)floorf((float)x2 * a.width_scale), (int)a.width1 - 1);
+      a.odata[index] = a.idata[(c * a.height1 + y1) * a.width1 + x1];
+    }
+  }
+};
+
+// ----------------------------------------------------------------------------
+// batch_norm_collect_statistics_kernel<InvStd,float,float,float,int>
+// (argument list: scripts/data/ml-event.csv:14).  One plane (channel) per block
+// iteration: per-thread Welford, Chan merges across the wavefront with DPP /
+// permute shuffles, one barrier, then a second wave-level merge.
+// ----------------------------------------------------------------------------
+struct Welford {
+  float n, mean, m2;
+};
+
+__device__ __forceinline__ Welford chan_merge(const Welford &a, const Welford &b) {
+  Welford r;
+  r.n = a.n + b.n;
+  const float f = r.n > 0.0f ? b.n * __frcp_rn(r.n) : 0.0f;
+  const float d = b.mean - a.mean;
+  r.mean = a.mean + d * f;
+  r.m2 = a.m2 + b.m2 + d * d * a.n * f;
+  return r;
+}
+
+// Butterfly over the 64 lanes.  The first four steps stay inside a row of 16
+// lanes and use DPP (quad permutes, half-row and row mirrors: the merge is
+// symmetric, so a mirror is as good as an xor); the last two cross rows.
+template <int CTRL>
+__device__ __forceinline__ float dpp(float v) {
+  return __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), CTRL, 0xF, 0xF, false));
+}
+template <int CTRL>
+__device__ __forceinline__ Welford dpp(const Welford &w) {
+  return Welford{dpp<CTRL>(w.n), dpp<CTRL>(w.mean), dpp<CTRL>(w.m2)};
+}
+__device__ __forceinline__ Welford shfl_xor(const Welford &w, int m) {
+  return Welford{__shfl_xor(w.n, m), __shfl_xor(w.mean, m), __shfl_xor(w.m2, m)};
+}
+__device__ __forceinline__ Welford wave_merge(Welford w) {
+  w = chan_merge(w, dpp<0xB1>(w));   // quad_perm [1,0,3,2]
+  w = chan_merge(w, dpp<0x4E>(w));   // quad_perm [2,3,0,1]
+  w = chan_merge(w, dpp<0x141>(w));  // row_half_mirror
+  w = chan_merge(w, dpp<0x140>(w));  // row_mirror
+  w = chan_merge(w, shfl_xor(w, 16));
+  w = chan_merge(w, shfl_xor(w, 32));
+  return w;
+}
+
+struct BnStatsBody {
+  using Args = hf_bn_stats_args;
+  static constexpr bool kBarriers = true;
+  static constexpr unsigned kLdsBytes = 16 * sizeof(Welford) + 16;
+
+  template <class SB>
+  static __device__ void run(const Args &a, SB &sb, unsigned char *lds, unsigned hint) {
+    Welford *part = reinterpret_cast<Welford *>(lds);
+    const int N = a.input.sizes[0], C = a.input.sizes[1], L = a.input.sizes[2];
+    for (int plane = (int)sb.bid; plane < C; plane += (int)sb.nblocks) {
+      Welford acc{0.0f, 0.0f, 0.0f};
+      if (hint == HINT_BN_VEC4) {
+        // stride[2] == 1, L % 4 == 0, 16-byte aligned rows: chunks of four.
+        const unsigned lq = (unsigned)L >> 2;
+        const unsigned chunks = (unsigned)N * lq;
+        const float *base = a.input.data + (size_t)plane * a.input.strides[1];
+        float k = 0.0f;
+        for (unsigned ch = sb.tid; ch < chunks; ch += sb.nthreads) {
+          const unsigned b = ch / lq, q = ch - b * lq;
+          const f32x4 v = ld4(base + (size_t)b * a.input.strides[0] + (size_t)q * 4);
+          // Welford of the chunk, then merge (4, m4, s4) into the running triple.
+          const float m4 = (v.x + v.y + v.z + v.w) * 0.25f;
+          const float dx = v.x - m4, dy = v.y - m4, dz = v.z - m4, dw = v.w - m4;
+          const float s4 = dx * dx + dy * dy + dz * dz + dw * dw;
+          k += 1.0f;
+          const float inv = __frcp_rn(k);           // 4 / (4k)
+          const float d = m4 - acc.mean;
+          acc.mean += d * inv;
+          acc.m2 += s4 + d * d * (4.0f * (k - 1.0f)) * inv;
+        }
+        acc.n = 4.0f * k;
+      } else {
+        const int total = N * L;
+        for (int e = (int)sb.tid; e < total; e += (int)sb.nthreads) {
+          const int b = e / L, x = e - b * L;
+          const float v = a.input.data[(size_t)b * a.input.strides[0] + (size_t)plane * a.input.strides[1] +
+                                       (size_t)x * a.input.strides[2]];
+          const float d1 = v - acc.mean;
+          acc.n += 1.0f;
+          acc.mean += d1 * __frcp_rn(acc.n);
+          acc.m2 += d1 * (v - acc.mean);
+        }
+      }
+      acc = wave_merge(acc);
+      if (sb.lane() == 0) part[sb.wave()] = acc;
+      sb.sync();
+      if (sb.wave() == 0) {
+        Welford w = sb.lane() < sb.nwaves() ? part[sb.lane()] : Welford{0.0f, 0.0f, 0.0f};
+        w = wave_merge(w);
+        if (sb.lane() == 0) {
+          a.save_mean.data[(size_t)plane * a.save_mean.strides[0]] = w.mean;
+          a.save_transformed_var.data[(size_t)plane * a.save_transformed_var.strides[0]] =
+              1.0f / sqrtf(w.m2 / w.n + a.epsilon);
+        }
+      }
+      sb.sync();  // the partial slots are reused by the next plane
+    }
+  }
+};
+
+// ----------------------------------------------------------------------------
+// kernelHistogram1D<..., SHARED, ...>  (argument list: scripts/data/ml-event.csv:2)
+// LDS bins, zero -> barrier -> grid-stride atomic accumulation -> barrier ->
+// flush to the fp32 counts with global atomics.
+// ----------------------------------------------------------------------------
+struct HistcBody {
+  using Args = hf_histc_args;
+  static constexpr bool kBarriers = true;
+
+  static __device__ __forceinline__ void count(unsigned *bins, float v, float lo, float hi, float scale_n, float range, int nbins) {
+    if (v >= lo && v <= hi) {
+      int bin = (int)((v - lo) * scale_n / range);
+      if (bin == nbins) bin -= 1;
+      __hip_atomic_fetch_add(bins + bin, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+    }
+  }
+
+  template <class SB>
+  static __device__ void run(const Args &a, SB &sb, unsigned char *lds, unsigned hint) {
+    unsigned *bins = reinterpret_cast<unsigned *>(lds);
+    const int nbins = a.nbins;
+    for (int i = (int)sb.tid; i < nbins; i += (int)sb.nthreads) bins[i] = 0;
+    sb.sync();
+    const float lo = a.minvalue, hi = a.maxvalue, range = hi - lo, fn = (float)nbins;
+    const float *b = a.b.data;
+    const int64_t total = a.total_elements;
+    if (hint == HINT_HIST_VEC4) {
+      const int64_t n4 = total >> 2;
+      const int64_t stride = (int64_t)sb.nblocks * sb.nthreads;
+      for (int64_t i = (int64_t)sb.bid * sb.nthreads + sb.tid; i < n4; i += stride) {
+        const f32x4 v = ld4(b + i * 4);
+        count(bins, v.x, lo, hi, fn, range, nbins);
+        count(bins, v.y, lo, hi, fn, range, nbins);
+        count(bins, v.z, lo, hi, fn, range, nbins);
+        count(bins, v.w, lo, hi, fn, range, nbins);
+      }
+      if (sb.bid == 0)
+        for (int64_t i = (n4 << 2) + sb.tid; i < total; i += sb.nthreads) count(bins, b[i], lo, hi, fn, range, nbins);
+    } else {
+      const int64_t stride = (int64_t)sb.nblocks * sb.nthreads;
+      const int64_t bs = a.b.strides[0];
+      for (int64_t i = (int64_t)sb.bid * sb.nthreads + sb.tid; i < total; i += stride)
+        count(bins, b[i * bs], lo, hi, fn, range, nbins);
+    }
+    sb.sync();
+    const int64_t as = a.a.strides[0];
+    for (int i = (int)sb.tid; i < nbins; i += (int)sb.nthreads) {
+      const unsigned c = bins[i];
+      if (c) unsafeAtomicAdd(a.a.data + i * as, (float)c);
+    }
+  }
+};
+
+}  // namespace hfuse

@@ -1,0 +1,127 @@
+// The view a kernel body has of "its" threads, whether it owns the whole
+// workgroup (native launch) or a wavefront-aligned slice of it (fused launch).
+//
+// The reference rewrites threadIdx/blockDim of each original kernel into
+// per-kernel locals computed from (flat tid - lower bound)
+// (lib/KernelFuser/ThreadInfoRewriter.cpp:38-58) and leaves blockIdx/gridDim
+// alone (include/ThreadInfoRewriter.h:29-31).  A body here is written once
+// against SubBlock and never touches threadIdx/blockDim itself.
+//
+// Barriers.  The reference turns __syncthreads() into the PTX named barrier
+// `bar.sync id,count` (lib/KernelFuser/BarrierRewriter.cpp:12-16) so a half
+// only waits for itself.  gfx950 has one barrier per workgroup (s_barrier
+// waits for every wave that has not ended), so a half that synchronises next to
+// a half that streams uses an LDS arrival counter instead: lane 0 of each wave
+// of the half adds 1 and spins (s_sleep) until the counter reaches
+// phase * waves_in_half.  The counter only grows, so no reset race exists; the
+// fused kernel zeroes it before one workgroup-wide s_barrier that every wave of
+// both halves executes exactly once on entry.
+#pragma once
+#include <hip/hip_runtime.h>
+
+namespace hfuse {
+
+typedef float f32x4 __attribute__((ext_vector_type(4)));
+typedef float f32x2 __attribute__((ext_vector_type(2)));
+typedef long long i64x2 __attribute__((ext_vector_type(2)));
+typedef unsigned int u32x4 __attribute__((ext_vector_type(4)));
+typedef unsigned int u32x2 __attribute__((ext_vector_type(2)));
+
+enum { BAR_WORKGROUP = 0, BAR_SUBSET = 1 };
+
+template <int BAR>
+struct SubBlock {
+  unsigned tid;       // thread index inside this half
+  unsigned nthreads;  // threads of this half (a multiple of 64)
+  unsigned bid;       // block index the body strides from
+  unsigned nblocks;   // grid size the body strides by
+  unsigned *bar;      // LDS arrival counter of this half (BAR_SUBSET only)
+  unsigned phase;     // barriers this thread has passed
+
+  __device__ __forceinline__ unsigned lane() const { return tid & 63u; }
+  __device__ __forceinline__ unsigned wave() const { return tid >> 6; }
+  __device__ __forceinline__ unsigned nwaves() const { return nthreads >> 6; }
+
+  __device__ __forceinline__ void sync() {
+    if constexpr (BAR == BAR_WORKGROUP) {
+      __syncthreads();
+    } else {
+      phase++;
+      // Release this wave's LDS/global writes to the workgroup, arrive, wait, acquire.
+      __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
+      if (lane() == 0) {
+        __hip_atomic_fetch_add(bar, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+        const unsigned target = phase * nwaves();
+        while (__hip_atomic_load(bar, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP) < target)
+          __builtin_amdgcn_s_sleep(1);
+      }
+      __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup");
+    }
+  }
+};
+
+// Launch geometry the host passes next to the two argument lists.
+struct FuseGeom {
+  unsigned d1, d2;          // threads of each half
+  unsigned lds1, lds2;      // LDS bytes of each half
+  unsigned hint1, hint2;    // fast-path selector the host derived from each argument list
+  unsigned grid1, grid2;    // blockIdx mode: workgroups given to each kernel
+};
+
+constexpr unsigned kBarrierWords = 4;  // 16 bytes reserved at the base of LDS for arrival counters
+
+// Native launch: the body owns the whole workgroup.
+template <class K, int T>
+__global__ __launch_bounds__(T) void native_kernel(typename K::Args a, unsigned hint) {
+  extern __shared__ __align__(16) unsigned char smem[];
+  SubBlock<BAR_WORKGROUP> sb{threadIdx.x, blockDim.x, blockIdx.x, gridDim.x, nullptr, 0};
+  K::run(a, sb, smem, hint);
+}
+
+// Horizontal fusion: waves [0, d1/64) run kernel 1, the rest run kernel 2.  The
+// selector is a scalar (readfirstlane) so each wave takes one side without
+// divergence.  MATCHED: both bodies execute the same number of barriers, so
+// they may share the hardware barrier; otherwise a body that synchronises
+// uses its own LDS counter.
+template <class K1, class K2, int T, bool MATCHED>
+__global__ __launch_bounds__(T) void fused_kernel(typename K1::Args a1, typename K2::Args a2, FuseGeom g) {
+  extern __shared__ __align__(16) unsigned char smem[];
+  unsigned *bars = reinterpret_cast<unsigned *>(smem);
+  const unsigned tid = threadIdx.x;
+  constexpr bool kSubset = !MATCHED && (K1::kBarriers || K2::kBarriers);
+  if constexpr (kSubset) {
+    if (tid < kBarrierWords) bars[tid] = 0;
+    __syncthreads();
+  }
+  const unsigned wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  constexpr int B1 = (kSubset && K1::kBarriers) ? BAR_SUBSET : BAR_WORKGROUP;
+  constexpr int B2 = (kSubset && K2::kBarriers) ? BAR_SUBSET : BAR_WORKGROUP;
+  if (wave < (g.d1 >> 6)) {
+    SubBlock<B1> sb{tid, g.d1, blockIdx.x, gridDim.x, bars + 0, 0};
+    K1::run(a1, sb, smem + 4 * kBarrierWords, g.hint1);
+  } else {
+    SubBlock<B2> sb{tid - g.d1, g.d2, blockIdx.x, gridDim.x, bars + 1, 0};
+    K2::run(a2, sb, smem + 4 * kBarrierWords + g.lds1, g.hint2);
+  }
+}
+
+// Fallback when the halves cannot share a workgroup: workgroups [0, grid1) run
+// kernel 1 and [grid1, grid1+grid2) run kernel 2, each with the whole
+// workgroup's hardware barrier.  The block is max(d1, d2) threads; waves beyond
+// a kernel's own size end at once (ended waves do not count at s_barrier).
+template <class K1, class K2, int T>
+__global__ __launch_bounds__(T) void blockidx_kernel(typename K1::Args a1, typename K2::Args a2, FuseGeom g) {
+  extern __shared__ __align__(16) unsigned char smem[];
+  const unsigned tid = threadIdx.x;
+  if (blockIdx.x < g.grid1) {
+    if (tid >= g.d1) return;
+    SubBlock<BAR_WORKGROUP> sb{tid, g.d1, blockIdx.x, g.grid1, nullptr, 0};
+    K1::run(a1, sb, smem, g.hint1);
+  } else {
+    if (tid >= g.d2) return;
+    SubBlock<BAR_WORKGROUP> sb{tid, g.d2, blockIdx.x - g.grid1, g.grid2, nullptr, 0};
+    K2::run(a2, sb, smem, g.hint2);
+  }
+}
+
+}  // namespace hfuse

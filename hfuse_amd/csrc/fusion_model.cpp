@@ -1,0 +1,256 @@
+#include "fusion_model.h"
+
+#include <algorithm>
+#include <cstdlib>
+
+#include "../../include/hfuse_gfx950.h"
+#include "yaml_lite.h"
+
+namespace hfuse {
+namespace {
+
+const Preset kPresets[] = {
+    // name        BaseLine BarSync LaunchBound ImBalanced   (main.cpp:182-193)
+    {"vfuse_lb", true, false, true, false},
+    {"vfuse", true, false, false, false},
+    {"hfuse", false, false, false, true},
+    {"hfuse_lb", false, false, true, true},
+};
+
+bool to_uint(const YamlNode *n, uint32_t &out) {
+  if (!n || n->kind != YamlNode::Scalar || n->scalar.empty()) return false;
+  char *end = nullptr;
+  unsigned long v = std::strtoul(n->scalar.c_str(), &end, 10);
+  if (*end != 0 || n->scalar[0] == '-') return false;
+  out = (uint32_t)v;
+  return true;
+}
+
+bool to_bool(const YamlNode *n, bool &out) {
+  if (!n || n->kind != YamlNode::Scalar) return false;
+  std::string s = n->scalar;
+  std::transform(s.begin(), s.end(), s.begin(), ::tolower);
+  if (s == "true" || s == "yes" || s == "on") { out = true; return true; }
+  if (s == "false" || s == "no" || s == "off") { out = false; return true; }
+  return false;
+}
+
+std::string at(const YamlNode &n) { return "line " + std::to_string(n.line) + ": "; }
+
+// One kernel row.  Map form: all of KernelName/HasBarriers/BlockDim/Reg are required
+// (KernelFusion.h:131-137); the older list form was written without Reg.
+bool parse_row(const YamlNode &n, bool reg_required, KernelRow &row, std::string &err) {
+  if (n.kind != YamlNode::Map) { err = at(n) + "kernel row must be a mapping"; return false; }
+  const YamlNode *name = n.get("KernelName");
+  if (!name || name->kind != YamlNode::Scalar || name->scalar.empty()) {
+    err = at(n) + "missing required key 'KernelName'";
+    return false;
+  }
+  row.name = name->scalar;
+  if (!to_bool(n.get("HasBarriers"), row.has_barriers)) {
+    err = at(n) + "missing or invalid required key 'HasBarriers'";
+    return false;
+  }
+  const YamlNode *bd = n.get("BlockDim");
+  if (!bd || bd->kind != YamlNode::Map || !to_uint(bd->get("X"), row.block_dim.x) ||
+      !to_uint(bd->get("Y"), row.block_dim.y) || !to_uint(bd->get("Z"), row.block_dim.z)) {
+    err = at(n) + "missing or invalid required key 'BlockDim' {X, Y, Z}";
+    return false;
+  }
+  const YamlNode *reg = n.get("Reg");
+  if (reg) {
+    if (!to_uint(reg, row.reg)) { err = at(n) + "invalid 'Reg'"; return false; }
+  } else if (reg_required) {
+    err = at(n) + "missing required key 'Reg'";
+    return false;
+  }
+  const YamlNode *et = n.get("ExecTime");
+  row.exec_time = -1.0;
+  if (et) {
+    char *end = nullptr;
+    row.exec_time = std::strtod(et->scalar.c_str(), &end);
+    if (et->kind != YamlNode::Scalar || et->scalar.empty() || *end != 0) {
+      err = at(n) + "invalid 'ExecTime'";
+      return false;
+    }
+  }
+  for (auto &kv : n.map) {
+    const std::string &k = kv.first;
+    if (k != "KernelName" && k != "HasBarriers" && k != "BlockDim" && k != "Reg" && k != "ExecTime") {
+      err = at(kv.second) + "unknown key '" + k + "'";
+      return false;
+    }
+  }
+  return true;
+}
+
+}  // namespace
+
+const KernelRow *Config::find(const std::string &key) const {
+  for (auto &r : rows)
+    if (r.key == key) return &r;
+  return nullptr;
+}
+
+const Preset *find_preset(const std::string &name) {
+  for (auto &p : kPresets)
+    if (name == p.name) return &p;
+  return nullptr;
+}
+
+bool parse_config(const char *fusion_yaml, const char *kernels_yaml, Config &cfg, std::string &err) {
+  cfg = Config();
+  if (!kernels_yaml) { err = "kernel table is null"; return false; }
+  YamlNode kroot;
+  if (!yaml_parse(kernels_yaml, kroot, err)) { err = "kernel table: " + err; return false; }
+  if (kroot.kind == YamlNode::Map) {
+    for (auto &kv : kroot.map) {
+      KernelRow row;
+      row.key = kv.first;
+      if (!parse_row(kv.second, true, row, err)) { err = "kernel table: " + err; return false; }
+      cfg.rows.push_back(row);
+    }
+  } else if (kroot.kind == YamlNode::Seq) {
+    for (auto &n : kroot.seq) {
+      KernelRow row;
+      if (!parse_row(n, false, row, err)) { err = "kernel table: " + err; return false; }
+      row.key = row.name;
+      if (cfg.find(row.key)) { err = "kernel table: duplicate kernel '" + row.key + "'"; return false; }
+      cfg.rows.push_back(row);
+    }
+  } else {
+    err = "kernel table: expected a mapping of kernels or a list of kernel rows";
+    return false;
+  }
+  if (cfg.rows.empty()) { err = "kernel table: no kernels"; return false; }
+
+  if (!fusion_yaml) {
+    if (kroot.kind != YamlNode::Seq) { err = "fusion list is null"; return false; }
+    FusionRow f;
+    for (auto &r : cfg.rows) f.kernels.push_back(r.key);
+    cfg.fusions.push_back(f);
+  } else {
+    YamlNode froot;
+    if (!yaml_parse(fusion_yaml, froot, err)) { err = "fusion list: " + err; return false; }
+    if (froot.kind != YamlNode::Seq) { err = "fusion list: expected a sequence of {File, Kernels}"; return false; }
+    for (auto &n : froot.seq) {
+      FusionRow f;
+      const YamlNode *file = n.kind == YamlNode::Map ? n.get("File") : nullptr;
+      const YamlNode *ks = n.kind == YamlNode::Map ? n.get("Kernels") : nullptr;
+      if (!file || file->kind != YamlNode::Scalar) { err = "fusion list: " + at(n) + "missing required key 'File'"; return false; }
+      if (!ks || ks->kind != YamlNode::Seq) { err = "fusion list: " + at(n) + "missing required key 'Kernels'"; return false; }
+      f.file = file->scalar;
+      for (auto &k : ks->seq) {
+        if (k.kind != YamlNode::Scalar) { err = "fusion list: " + at(k) + "kernel name must be a scalar"; return false; }
+        f.kernels.push_back(k.scalar);
+      }
+      cfg.fusions.push_back(f);
+    }
+  }
+  for (auto &f : cfg.fusions) {
+    if (f.kernels.size() != 2) { err = "fusion '" + f.file + "': exactly two kernels are fused"; return false; }
+    for (auto &k : f.kernels)
+      if (!cfg.find(k)) { err = "fusion '" + f.file + "': kernel '" + k + "' is not in the kernel table"; return false; }
+  }
+  return true;
+}
+
+int num_splits(const KernelRow &k1, const KernelRow &k2) {
+  uint32_t end = k1.block_dim.size() + k2.block_dim.size();
+  int n = 0;
+  for (uint32_t split = 128; split < end; split += 128) n++;
+  return n;
+}
+
+int make_partition(const KernelRow &k1, const KernelRow &k2, const Preset &preset, int split_idx,
+                   int split_threads, Partition &out, std::string &err) {
+  const KernelRow *rows[2] = {&k1, &k2};
+  Dim3 dims[2] = {k1.block_dim, k2.block_dim};
+  const uint32_t total = dims[0].size() + dims[1].size();
+  if (dims[0].size() == 0 || dims[1].size() == 0) { err = "empty BlockDim"; return HF_EINVAL; }
+  std::string variant = preset.name;
+
+  if (!preset.base_line) {
+    uint32_t first = dims[0].size();
+    bool resplit = false;
+    if (split_threads > 0) {
+      first = (uint32_t)split_threads;
+      resplit = true;
+      variant += "_split_" + std::to_string(first);
+    } else if (split_idx >= 0 || split_idx == HF_SPLIT_EXECTIME) {
+      // Context's imbalanced re-split (KernelFusion.h:63-72) with the wavefront as granule.
+      double e0, e1;
+      if (split_idx >= 0) {
+        if (split_idx >= num_splits(k1, k2)) { err = "split index beyond the enumeration 128*(n+1) < d1+d2"; return HF_EINVAL; }
+        e0 = 128.0 * (split_idx + 1);  // main.cpp:224-225
+        e1 = (double)total - e0;
+        variant += "_idx_" + std::to_string(split_idx);
+      } else {
+        e0 = k1.exec_time;
+        e1 = k2.exec_time;
+        if (!(e0 > 0) || !(e1 > 0)) { err = "ExecTime split requested but the table has no ExecTime"; return HF_EINVAL; }
+        variant += "_exectime";
+      }
+      first = (uint32_t)((int)(e0 / (e0 + e1) * total / kWave)) * kWave;
+      resplit = true;
+    } else {
+      variant += "_table";
+    }
+    if (resplit) {
+      if (first == 0 || first >= total) { err = "split leaves one kernel without threads"; return HF_EINVAL; }
+      uint32_t parts[2] = {first, total - first};
+      for (int i = 0; i < 2; i++) {
+        if (dims[i].y == 0 || dims[i].z != 1 || parts[i] % dims[i].y != 0) {
+          err = "split of " + std::to_string(parts[i]) + " threads does not divide by BlockDim.Y of '" + rows[i]->name + "'";
+          return HF_EINVAL;
+        }
+        dims[i].x = parts[i] / dims[i].y;  // KernelFusion.h:72
+      }
+    }
+    for (int i = 0; i < 2; i++) {
+      if (dims[i].size() % kWave != 0) {
+        err = "part of '" + rows[i]->name + "' is " + std::to_string(dims[i].size()) + " threads: not a multiple of the 64-lane wavefront";
+        return HF_EINVAL;
+      }
+    }
+    if (dims[0].size() + dims[1].size() > kMaxBlock) {
+      err = "fused block of " + std::to_string(dims[0].size() + dims[1].size()) + " threads exceeds 1024";
+      return HF_EINVAL;
+    }
+  } else {
+    variant += "_idx_0";  // main.cpp:218-219,223: the vertical presets print one variant
+    if (std::max(dims[0].size(), dims[1].size()) > kMaxBlock) { err = "block exceeds 1024 threads"; return HF_EINVAL; }
+  }
+
+  uint32_t b = 0;
+  for (int i = 0; i < 2; i++) {
+    out.lo[i] = b;
+    out.hi[i] = b + dims[i].size();
+    out.block_dim[i] = dims[i];
+    if (!preset.base_line) b += dims[i].size();  // KernelFusion.h:76-78
+  }
+  // KernelPrinter.cpp:46-66
+  uint32_t max_thread = 0, max_block = 9999999u, sum = 0;
+  for (int i = 0; i < 2; i++) {
+    uint32_t size = dims[i].size();
+    if (rows[i]->reg) max_block = std::min(kRegFile / rows[i]->reg / size, max_block);
+    sum += size;
+    max_thread = std::max(max_thread, size);
+  }
+  max_block = std::min(max_block, kMaxResidentThreads / sum);
+  out.launch_threads = preset.base_line ? max_thread : sum;
+  out.launch_blocks = preset.launch_bound ? max_block : 0;
+  out.name = k1.name + "_" + k2.name + "_fused_kernel_" + variant;  // KernelPrinter.cpp:67-70
+  return HF_OK;
+}
+
+Dim3 local_index(uint32_t tid, uint32_t lo, const Dim3 &dim) {
+  uint32_t t = tid - lo;
+  Dim3 r;
+  r.x = t % dim.x;
+  r.y = t / dim.x % dim.y;
+  r.z = t / (dim.x * dim.y);
+  return r;
+}
+
+}  // namespace hfuse

@@ -1,0 +1,74 @@
+// Host-side model of a horizontal fusion: the kernel table, the fusion list and
+// the thread partition of one fused variant.  Restates, for 64-lane wavefronts,
+// the rules of the reference's Context (include/KernelFusion.h:35-92), its split
+// enumeration (tools/llvm-smart-fuser/main.cpp:182-227) and the signature
+// printer (lib/KernelFuser/KernelPrinter.cpp:42-70).
+#pragma once
+#include <cstdint>
+#include <map>
+#include <string>
+#include <vector>
+
+namespace hfuse {
+
+struct Dim3 {
+  uint32_t x = 1, y = 1, z = 1;
+  uint32_t size() const { return x * y * z; }
+};
+
+struct KernelRow {
+  std::string key;   // map key (or KernelName in the list form)
+  std::string name;  // KernelName
+  bool has_barriers = false;
+  Dim3 block_dim;
+  uint32_t reg = 0;
+  double exec_time = -1.0;
+};
+
+struct FusionRow {
+  std::string file;
+  std::vector<std::string> kernels;
+};
+
+struct Config {
+  std::vector<KernelRow> rows;  // table order
+  std::vector<FusionRow> fusions;
+  const KernelRow *find(const std::string &key) const;
+};
+
+// The four presets of main.cpp:182-193 as {BaseLine, BarSync, LaunchBound, ImBalancedThread}.
+struct Preset {
+  const char *name;
+  bool base_line, bar_sync, launch_bound, imbalanced;
+};
+const Preset *find_preset(const std::string &name);
+
+struct Partition {
+  uint32_t lo[2], hi[2];
+  Dim3 block_dim[2];
+  uint32_t launch_threads = 0, launch_blocks = 0;
+  std::string name;  // <K1>_<K2>_fused_kernel_<preset>_idx_<n>
+};
+
+// gfx950 constants standing in for KernelPrinter.cpp:10-11 (64K registers, 2048 threads per SM):
+// one CU holds 4 SIMDs x 512 VGPRs x 64 lanes and at most 2048 resident work-items.
+constexpr uint32_t kRegFile = 4 * 512 * 64;
+constexpr uint32_t kMaxResidentThreads = 2048;
+constexpr uint32_t kWave = 64;
+constexpr uint32_t kMaxBlock = 1024;
+
+bool parse_config(const char *fusion_yaml, const char *kernels_yaml, Config &cfg, std::string &err);
+
+// Number of variants the split loop prints for a horizontal preset (main.cpp:221-223).
+int num_splits(const KernelRow &k1, const KernelRow &k2);
+
+// split_threads > 0: explicit size of kernel 1's part; else split_idx >= 0: the reference's
+// enumeration (Split = 128*(idx+1)); else (-1) the table's own BlockDim.
+// Returns 0, or a negative HF_E* code with `err` set.
+int make_partition(const KernelRow &k1, const KernelRow &k2, const Preset &preset, int split_idx,
+                   int split_threads, Partition &out, std::string &err);
+
+// ThreadInfoRewriter.cpp:38-58
+Dim3 local_index(uint32_t tid, uint32_t lo, const Dim3 &dim);
+
+}  // namespace hfuse

@@ -1,0 +1,70 @@
+// Instantiations of the nonce-search kernels: four native kernels and the
+// ordered pairs of the reference's crypto_fusion.yaml (both orders).
+#include "device/crypto_bodies.h"
+#include "launch.h"
+
+namespace hfuse {
+namespace {
+
+// The searches run 128+128 threads in the reference's YAML; 512 leaves room for
+// every 64-lane re-split of up to 512 threads.  Four waves per SIMD keeps each
+// wave under 128 VGPRs so a memory-bound half still has waves to hide latency.
+constexpr int kCryptoBlock = 512;
+
+template <class K>
+hipError_t native(const void *args, unsigned hint, unsigned grid, unsigned block, size_t lds, hipStream_t s) {
+  hipLaunchKernelGGL((native_kernel<K, kCryptoBlock>), dim3(grid), dim3(block), lds, s,
+                     *static_cast<const typename K::Args *>(args), hint);
+  return hipGetLastError();
+}
+
+template <class K1, class K2>
+hipError_t pair(FuseMode mode, const void *a1, const void *a2, const FuseGeom &g, unsigned grid, size_t lds,
+                hipStream_t s) {
+  const auto &x1 = *static_cast<const typename K1::Args *>(a1);
+  const auto &x2 = *static_cast<const typename K2::Args *>(a2);
+  if (g.d1 + g.d2 > (unsigned)kCryptoBlock) return hipErrorNotSupported;
+  switch (mode) {
+    case MODE_HFUSE:
+      hipLaunchKernelGGL((fused_kernel<K1, K2, kCryptoBlock, false>), dim3(grid), dim3(g.d1 + g.d2), lds, s, x1, x2,
+                         g);
+      break;
+    case MODE_MATCHED:
+      return hipErrorNotSupported;  // none of the searches has a barrier
+    case MODE_BLOCKIDX:
+      hipLaunchKernelGGL((blockidx_kernel<K1, K2, kCryptoBlock>), dim3(grid), dim3(g.d1 > g.d2 ? g.d1 : g.d2), lds,
+                         s, x1, x2, g);
+      break;
+  }
+  return hipGetLastError();
+}
+
+}  // namespace
+
+hipError_t launch_native_crypto(KernelId k, const void *args, unsigned hint, unsigned grid, unsigned block, size_t lds,
+                                hipStream_t s) {
+  switch (k) {
+    case K_ETHASH: return native<EthashBody>(args, hint, grid, block, lds, s);
+    case K_SHA256D: return native<Sha256dBody>(args, hint, grid, block, lds, s);
+    case K_SIA_BLAKE2B: return native<SiaBlake2bBody>(args, hint, grid, block, lds, s);
+    case K_BLAKE2B: return native<CcminerBlake2bBody>(args, hint, grid, block, lds, s);
+    default: return hipErrorNotSupported;
+  }
+}
+
+#define HF_PAIR(A, KA, B, KB)                                                     \
+  if (k1 == A && k2 == B) return pair<KA, KB>(mode, a1, a2, g, grid, lds, s);     \
+  if (k1 == B && k2 == A) return pair<KB, KA>(mode, a1, a2, g, grid, lds, s);
+
+hipError_t launch_fused_crypto(KernelId k1, KernelId k2, FuseMode mode, const void *a1, const void *a2,
+                               const FuseGeom &g, unsigned grid, size_t lds, hipStream_t s) {
+  HF_PAIR(K_ETHASH, EthashBody, K_BLAKE2B, CcminerBlake2bBody)
+  HF_PAIR(K_SHA256D, Sha256dBody, K_ETHASH, EthashBody)
+  HF_PAIR(K_SIA_BLAKE2B, SiaBlake2bBody, K_ETHASH, EthashBody)
+  HF_PAIR(K_BLAKE2B, CcminerBlake2bBody, K_SHA256D, Sha256dBody)
+  HF_PAIR(K_BLAKE2B, CcminerBlake2bBody, K_SIA_BLAKE2B, SiaBlake2bBody)
+  HF_PAIR(K_SHA256D, Sha256dBody, K_SIA_BLAKE2B, SiaBlake2bBody)
+  return hipErrorNotSupported;
+}
+
+}  // namespace hfuse

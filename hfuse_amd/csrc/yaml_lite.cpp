@@ -1,0 +1,173 @@
+#include "yaml_lite.h"
+
+#include <sstream>
+
+namespace hfuse {
+namespace {
+
+struct Line {
+  int indent;
+  std::string text;  // without indent, comments and trailing blanks
+  int no;
+};
+
+std::string rstrip(std::string s) {
+  while (!s.empty() && (s.back() == ' ' || s.back() == '\t' || s.back() == '\r')) s.pop_back();
+  return s;
+}
+
+std::string strip_comment(const std::string &s) {
+  bool sq = false, dq = false;
+  for (size_t i = 0; i < s.size(); i++) {
+    char c = s[i];
+    if (c == '\'' && !dq) sq = !sq;
+    if (c == '"' && !sq) dq = !dq;
+    if (c == '#' && !sq && !dq && (i == 0 || s[i - 1] == ' ' || s[i - 1] == '\t')) return s.substr(0, i);
+  }
+  return s;
+}
+
+std::string unquote(std::string s) {
+  s = rstrip(s);
+  size_t b = 0;
+  while (b < s.size() && s[b] == ' ') b++;
+  s = s.substr(b);
+  if (s.size() >= 2 && ((s.front() == '"' && s.back() == '"') || (s.front() == '\'' && s.back() == '\'')))
+    return s.substr(1, s.size() - 2);
+  return s;
+}
+
+// Position of the ':' that ends a mapping key ("key: v" or "key:"), or npos.
+size_t key_colon(const std::string &t) {
+  bool sq = false, dq = false;
+  for (size_t i = 0; i < t.size(); i++) {
+    char c = t[i];
+    if (c == '\'' && !dq) sq = !sq;
+    if (c == '"' && !sq) dq = !dq;
+    if (c == ':' && !sq && !dq && (i + 1 == t.size() || t[i + 1] == ' ')) return i;
+  }
+  return std::string::npos;
+}
+
+bool is_seq_item(const std::string &t) { return t == "-" || (t.size() >= 2 && t[0] == '-' && t[1] == ' '); }
+
+struct Parser {
+  std::vector<Line> lines;
+  size_t pos = 0;
+  std::string err;
+
+  bool fail(int no, const std::string &why) {
+    std::ostringstream o;
+    o << "line " << no << ": " << why;
+    err = o.str();
+    return false;
+  }
+
+  bool parse_block(int indent, YamlNode &out) {
+    if (pos >= lines.size()) return true;
+    if (is_seq_item(lines[pos].text)) return parse_seq(indent, out);
+    return parse_map(indent, out);
+  }
+
+  bool parse_seq(int indent, YamlNode &out) {
+    out.kind = YamlNode::Seq;
+    out.line = lines[pos].no;
+    while (pos < lines.size() && lines[pos].indent == indent && is_seq_item(lines[pos].text)) {
+      Line &ln = lines[pos];
+      std::string rest = ln.text.size() > 1 ? ln.text.substr(1) : "";
+      size_t skip = 0;
+      while (skip < rest.size() && rest[skip] == ' ') skip++;
+      rest = rest.substr(skip);
+      YamlNode item;
+      item.line = ln.no;
+      if (rest.empty()) {
+        pos++;
+        if (pos < lines.size() && lines[pos].indent > indent) {
+          if (!parse_block(lines[pos].indent, item)) return false;
+        }
+      } else if (key_colon(rest) != std::string::npos) {
+        // "- key: value": the map starts on the dash line, at the column of `key`.
+        int child = indent + 1 + (int)skip;
+        ln.indent = child;
+        ln.text = rest;
+        if (!parse_map(child, item)) return false;
+      } else {
+        item.kind = YamlNode::Scalar;
+        item.scalar = unquote(rest);
+        pos++;
+      }
+      out.seq.push_back(std::move(item));
+    }
+    if (pos < lines.size() && lines[pos].indent > indent) return fail(lines[pos].no, "unexpected indentation");
+    return true;
+  }
+
+  bool parse_map(int indent, YamlNode &out) {
+    out.kind = YamlNode::Map;
+    out.line = lines[pos].no;
+    while (pos < lines.size() && lines[pos].indent == indent && !is_seq_item(lines[pos].text)) {
+      const Line ln = lines[pos];
+      size_t c = key_colon(ln.text);
+      if (c == std::string::npos) return fail(ln.no, "expected 'key: value'");
+      std::string key = unquote(ln.text.substr(0, c));
+      std::string val = ln.text.substr(c + 1);
+      if (out.get(key)) return fail(ln.no, "duplicate key '" + key + "'");
+      YamlNode child;
+      child.line = ln.no;
+      pos++;
+      if (unquote(val).empty()) {
+        if (pos < lines.size() && lines[pos].indent > indent) {
+          if (!parse_block(lines[pos].indent, child)) return false;
+        } else if (pos < lines.size() && lines[pos].indent == indent && is_seq_item(lines[pos].text)) {
+          if (!parse_seq(indent, child)) return false;  // sequence at the key's own column
+        }
+      } else {
+        child.kind = YamlNode::Scalar;
+        child.scalar = unquote(val);
+        if (pos < lines.size() && lines[pos].indent > indent)
+          return fail(lines[pos].no, "unexpected indentation after scalar value");
+      }
+      out.map.emplace_back(std::move(key), std::move(child));
+    }
+    return true;
+  }
+};
+
+}  // namespace
+
+bool yaml_parse(const std::string &text, YamlNode &root, std::string &err) {
+  Parser p;
+  std::istringstream in(text);
+  std::string raw;
+  int no = 0;
+  while (std::getline(in, raw)) {
+    no++;
+    if (raw.find('\t') != std::string::npos && raw.find_first_not_of(" \t") != std::string::npos &&
+        raw.substr(0, raw.find_first_not_of(" \t")).find('\t') != std::string::npos) {
+      std::ostringstream o;
+      o << "line " << no << ": tab in indentation";
+      err = o.str();
+      return false;
+    }
+    std::string s = rstrip(strip_comment(raw));
+    size_t b = s.find_first_not_of(' ');
+    if (b == std::string::npos) continue;
+    if (s.compare(b, 3, "---") == 0 && rstrip(s.substr(b)) == "---") continue;
+    p.lines.push_back({(int)b, s.substr(b), no});
+  }
+  root = YamlNode();
+  if (p.lines.empty()) return true;
+  if (!p.parse_block(p.lines[0].indent, root)) {
+    err = p.err;
+    return false;
+  }
+  if (p.pos != p.lines.size()) {
+    std::ostringstream o;
+    o << "line " << p.lines[p.pos].no << ": inconsistent indentation";
+    err = o.str();
+    return false;
+  }
+  return true;
+}
+
+}  // namespace hfuse

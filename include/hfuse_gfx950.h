@@ -1,0 +1,318 @@
+/*
+ * hfuse_gfx950.h -- C-ABI of the MI355X (gfx950) horizontally fused kernel library.
+ *
+ * The reference (aoli-al/HFuse) is a source rewriter: its interface for this
+ * path is (1) two YAML files, (2) the name / thread partition / argument order
+ * of the fused kernel it prints, and (3) the argument lists of the original
+ * kernels.  This header is what an external host program binds instead of
+ * including the generated `<K1>_<K2>_.inc` text:
+ *
+ *   - hf_config_*   : the fusion list and kernel table
+ *                     (include/KernelFusion.h:129-159, configs/ml_fusion.yaml,
+ *                      configs/ml_kernels.yaml, configs/crypto_*.yaml)
+ *   - hf_plan_*     : one fused variant = pair x preset x split
+ *                     (include/KernelFusion.h:45-80,
+ *                      tools/llvm-smart-fuser/main.cpp:182-193,215-227,
+ *                      lib/KernelFuser/KernelPrinter.cpp:42-70)
+ *   - hf_*_args     : each original kernel's argument list, field for field
+ *                     (scripts/data/ml-event.csv, scripts/data/ethminer_event.csv)
+ *   - hf_launch_*   : native launch of one kernel, and the fused launch taking
+ *                     kernel 1's arguments then kernel 2's
+ *                     (lib/KernelFuser/KernelPrinter.cpp:107-115,
+ *                      scripts/configs/hist_norm.json:5)
+ *
+ * All pointers inside argument structs are caller-owned device memory; the
+ * library allocates no device memory.  Every call returns 0 or a negative
+ * HF_E* code and never throws; hf_last_error() gives the text for the calling
+ * thread.  Launches are asynchronous on the caller's hipStream_t (passed as
+ * void*; NULL is the default stream).
+ */
+#ifndef HFUSE_GFX950_H
+#define HFUSE_GFX950_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define HF_API __attribute__((visibility("default")))
+
+/* ------------------------------------------------------------------ errors */
+enum {
+  HF_OK = 0,
+  HF_EINVAL = -1,      /* bad argument (null pointer, bad shape, bad split ...) */
+  HF_EPARSE = -2,      /* YAML does not follow the reference schema            */
+  HF_ENOTFOUND = -3,   /* unknown kernel / pair / preset                       */
+  HF_EUNSUPPORTED = -4,/* legal in the reference, not built here               */
+  HF_EHIP = -5,        /* a HIP runtime call failed                            */
+  HF_EIO = -6          /* file could not be read                               */
+};
+
+HF_API const char *hf_last_error(void);
+HF_API int hf_version(void);
+
+/* ------------------------------------------------------------ configuration */
+typedef struct hf_config hf_config;
+
+typedef struct {
+  uint32_t x, y, z;
+} hf_dim3;
+
+/* One row of the kernel table: include/KernelFusion.h:21-27,129-138. */
+typedef struct {
+  char kernel_name[96];
+  int has_barriers;
+  hf_dim3 block_dim;
+  uint32_t reg;
+  double exec_time; /* -1 when the YAML has no ExecTime */
+} hf_kernel_info;
+
+/*
+ * Parse the two YAML documents of the reference's CLI
+ * (tools/llvm-smart-fuser/main.cpp:263-270): a sequence of {File, Kernels}
+ * and a string-keyed map of kernel rows.  `kernels_yaml` may also be the older
+ * per-pair form, a bare sequence of rows (configs/im2col_maxpool.yaml); then
+ * `fusion_yaml` may be NULL and the single fusion is that list in order.
+ */
+HF_API int hf_config_load_text(const char *fusion_yaml, const char *kernels_yaml, hf_config **out);
+HF_API int hf_config_load_files(const char *fusion_path, const char *kernels_path, hf_config **out);
+HF_API void hf_config_free(hf_config *cfg);
+HF_API int hf_config_num_fusions(const hf_config *cfg);
+HF_API int hf_config_num_kernels(const hf_config *cfg);
+/* Names of the i-th fusion's kernels (NUL-terminated, valid while cfg lives). */
+HF_API int hf_config_fusion(const hf_config *cfg, int i, const char **file, const char **k1,
+                            const char **k2);
+HF_API int hf_config_kernel(const hf_config *cfg, const char *name, hf_kernel_info *out);
+
+/* ------------------------------------------------------------------- plans */
+typedef struct hf_plan hf_plan;
+
+/*
+ * What the Context constructor and the printer decide for one variant
+ * (include/KernelFusion.h:45-80, lib/KernelFuser/KernelPrinter.cpp:42-70).
+ */
+typedef struct {
+  char name[256];          /* <K1>_<K2>_fused_kernel_<preset>_idx_<n>           */
+  uint32_t lo[2], hi[2];   /* thread bounds of each kernel inside the block      */
+  hf_dim3 block_dim[2];    /* per-kernel block shape after the re-split          */
+  uint32_t launch_threads; /* d1+d2 (hfuse) or max(d1,d2) (vfuse)                */
+  uint32_t launch_blocks;  /* min-blocks hint, 0 when the preset has none        */
+  int barrier_mode;        /* HF_BARRIER_* chosen for this pair                  */
+} hf_partition;
+
+enum {
+  HF_BARRIER_NONE = 0,     /* neither half synchronises                          */
+  HF_BARRIER_MATCHED = 1,  /* both halves execute the same s_barrier sequence    */
+  HF_BARRIER_SUBSET = 2,   /* LDS-counter barrier among one half's wavefronts    */
+  HF_BARRIER_BLOCKIDX = 3  /* fallback: halves live in different workgroups      */
+};
+
+#define HF_SPLIT_TABLE (-1)
+#define HF_SPLIT_EXECTIME (-2)
+#define HF_WAVE 64         /* split granularity (reference: 32, KernelFusion.h:66) */
+#define HF_MAX_BLOCK 1024
+
+/*
+ * Create a plan for fusion `fusion_index` of `cfg`.
+ *   preset    : "hfuse" | "hfuse_lb" | "vfuse" | "vfuse_lb" (main.cpp:182-193).
+ *               Fused launches are built for the two hfuse presets; the vfuse
+ *               presets only report their partition (launch returns
+ *               HF_EUNSUPPORTED).
+ *   split_idx : the reference's enumeration index n (Split = 128*(n+1) threads
+ *               for kernel 1, main.cpp:216-227); HF_SPLIT_TABLE keeps the
+ *               YAML's BlockDim as the split; HF_SPLIT_EXECTIME re-splits in
+ *               proportion to the table's ExecTime (KernelFusion.h:63-72).
+ *   split_threads : when > 0 overrides split_idx with an explicit thread count
+ *               for kernel 1 (must be a multiple of 64).
+ * Both parts must be non-empty multiples of 64 and d1+d2 <= 1024.
+ */
+HF_API int hf_plan_create(const hf_config *cfg, int fusion_index, const char *preset, int split_idx,
+                          int split_threads, hf_plan **out);
+HF_API void hf_plan_free(hf_plan *plan);
+/*
+ * Override the barrier design of a plan (HF_BARRIER_*).  The default is
+ * HF_BARRIER_NONE when neither body synchronises and HF_BARRIER_SUBSET when
+ * one does.  HF_BARRIER_MATCHED is legal when both bodies synchronise (they
+ * then share the hardware barrier); HF_BARRIER_BLOCKIDX is always legal.
+ */
+HF_API int hf_plan_set_barrier_mode(hf_plan *plan, int mode);
+HF_API int hf_plan_partition(const hf_plan *plan, hf_partition *out);
+/* Number of variants the reference's split loop would print (main.cpp:221-223). */
+HF_API int hf_plan_num_splits(const hf_config *cfg, int fusion_index);
+/* Local (x,y,z) of flat thread `tid` in half `half`: ThreadInfoRewriter.cpp:38-58. */
+HF_API int hf_plan_local_index(const hf_plan *plan, int half, uint32_t tid, hf_dim3 *out);
+
+/* ------------------------------------------------- original argument lists */
+
+/* im2col_kernel<float> -- scripts/data/ml-event.csv:17 */
+typedef struct {
+  int64_t n;
+  const float *data_im;
+  int64_t height, width, kernel_h, kernel_w, pad_h, pad_w, stride_h, stride_w, dilation_h,
+      dilation_w, height_col, width_col;
+  float *data_col;
+} hf_im2col_args;
+
+/* MaxPoolForward<float,float> -- scripts/data/ml-event.csv:5 */
+typedef struct {
+  int nthreads;
+  const float *bottom_data;
+  int num, channels, height, width, pooled_height, pooled_width, kernel_h, kernel_w, stride_h,
+      stride_w, pad_h, pad_w, dilation_h, dilation_w;
+  float *top_data;
+  int64_t *top_mask;
+} hf_maxpool_args;
+
+/* PackedTensorAccessor<float,N,...,int> flattened to {ptr, sizes, strides}. */
+typedef struct {
+  float *data;
+  int sizes[3];
+  int strides[3];
+} hf_accessor3;
+typedef struct {
+  float *data;
+  int sizes[1];
+  int strides[1];
+} hf_accessor1;
+
+/*
+ * batch_norm_collect_statistics_kernel<InvStd,float,float,float,int>
+ * -- scripts/data/ml-event.csv:14, call text scripts/configs/hist_norm.json:5.
+ * running_mean / running_var / momentum are accepted and ignored, as in the
+ * reference's call (dummy tensors, momentum 0.0).
+ */
+typedef struct {
+  hf_accessor3 input; /* [N, C, L] */
+  float epsilon;
+  float momentum;
+  hf_accessor1 running_mean, running_var, save_mean, save_transformed_var;
+} hf_bn_stats_args;
+
+/*
+ * upsample_nearest2d_out_frame<float> (PyTorch).  The reference fuses the
+ * bilinear kernel (configs/ml_kernels.yaml:1-9); this build's contract asks for
+ * nearest, whose argument list is the one below.
+ */
+typedef struct {
+  const float *idata;
+  float *odata;
+  size_t nc, height1, width1, height2, width2;
+  float height_scale, width_scale;
+} hf_upsample_nearest_args;
+
+/* cuda::detail::TensorInfo<float,long> flattened. */
+#define HF_MAX_TENSORINFO_DIMS 8
+typedef struct {
+  float *data;
+  int64_t sizes[HF_MAX_TENSORINFO_DIMS];
+  int64_t strides[HF_MAX_TENSORINFO_DIMS];
+  int dims;
+} hf_tensorinfo;
+
+/*
+ * kernelHistogram1D<float,float,long,1,2,-1,SHARED,Op>
+ * -- scripts/data/ml-event.csv:2, call text scripts/configs/hist_norm.json:5.
+ * a = output counts (fp32, caller-zeroed, accumulated with atomics),
+ * p = partial output (unused in SHARED mode), b = input.  getOp is the
+ * constant-1 functor of histc; a NULL function pointer slot keeps the arity.
+ * Only contiguous 1-D `a` and `b` are built (HF_EUNSUPPORTED otherwise).
+ */
+typedef struct {
+  hf_tensorinfo a, p, b;
+  int nbins;
+  float minvalue, maxvalue;
+  int64_t total_elements;
+  const void *get_op;
+} hf_histc_args;
+
+/* Search results shared by the three nonce searches (layout is this library's own). */
+#define HF_MAX_SEARCH_RESULTS 64
+typedef struct {
+  uint64_t nonce;     /* sha256d: 32-bit nonce; sia: the 8-byte word at offset 32; ethash: nonce */
+  uint32_t digest[8]; /* the 32 digest bytes as they lie in memory                               */
+  uint32_t mix[8];    /* ethash mix digest, zero otherwise                                       */
+} hf_search_hit;
+typedef struct {
+  uint32_t count;     /* total hits found (may exceed the recorded slots)                        */
+  uint32_t pad;
+  hf_search_hit hit[HF_MAX_SEARCH_RESULTS]; /* unordered; callers sort by nonce                  */
+} hf_search_results;
+
+/* ethash_search(volatile Search_results*, uint64_t) -- scripts/data/ethminer_event.csv:9 */
+typedef struct {
+  hf_search_results *g_output;
+  uint64_t start_nonce;
+} hf_ethash_args;
+
+/* sha256d_gpu_hash_shared(uint32, uint32, uint32*) -- scripts/data/ethminer_event.csv:26 */
+typedef struct {
+  uint32_t threads;
+  uint32_t start_nonce;
+  uint32_t *res_nonces; /* points at an hf_search_results */
+} hf_sha256d_args;
+
+/* sia_blake2b_gpu_hash / blake2b_gpu_hash(uint32, uint32, uint32*, uint2)
+ * -- scripts/data/ethminer_event.csv:2,22 */
+typedef struct {
+  uint32_t threads;
+  uint32_t start_nonce;
+  uint32_t *res_nonce; /* points at an hf_search_results */
+  uint32_t target2[2]; /* uint2: {low, high} words of the 64-bit target */
+} hf_blake2b_args;
+
+/*
+ * Constants the original kernels read from __constant__ symbols set by their
+ * host program.  Each call copies to this library's own device symbols on
+ * `stream`; they hold until the next call.
+ */
+/* ethash: DAG of 128-byte items, 32-byte header hash, 64-bit target. */
+HF_API int hf_ethash_set_constants(const void *dag, uint32_t dag_items, const uint8_t header[32],
+                                   uint64_t target, void *stream);
+/* sha256d: 80-byte header (nonce bytes 76..79 ignored) and the top 64 bits of
+ * the little-endian 256-bit target. */
+HF_API int hf_sha256d_set_block(const uint8_t header[80], uint64_t target64, void *stream);
+/* sia blake2b / ccminer blake2b: 80-byte header. */
+HF_API int hf_sia_blake2b_set_block(const uint8_t header[80], void *stream);
+HF_API int hf_blake2b_set_block(const uint8_t header[80], void *stream);
+
+/* ----------------------------------------------------------------- launches */
+/*
+ * Native launch of one original kernel by its YAML name; `args` points at the
+ * matching hf_*_args.  grid_blocks <= 0 lets the library size the grid from the
+ * work; block threads come from block_threads (<= 0: the kernel's default).
+ */
+HF_API int hf_launch_native(const char *kernel_name, const void *args, int grid_blocks,
+                            int block_threads, void *stream);
+/*
+ * Fused launch: one kernel whose workgroup is [0,d1) running kernel 1's body
+ * and [d1,d1+d2) running kernel 2's, arguments in YAML order
+ * (KernelPrinter.cpp:107-115).  grid_blocks <= 0: sized by the library.
+ */
+HF_API int hf_launch_fused(const hf_plan *plan, const void *args1, const void *args2,
+                           int grid_blocks, void *stream);
+
+/*
+ * Timing helper used by the benchmark: runs `iters` repetitions of
+ *   mode 0: native kernel 1      mode 1: native kernel 2
+ *   mode 2: kernel 1 then kernel 2 back to back on `stream`
+ *   mode 3: the fused kernel
+ * cycling through `nsets` argument sets (args1[i], args2[i]) so repeats do not
+ * hit in the last-level cache, and returns the elapsed milliseconds measured
+ * with HIP events recorded on `stream` around the timed launches.
+ */
+HF_API int hf_time_pair(const hf_plan *plan, int mode, const void *const *args1,
+                        const void *const *args2, int nsets, int warmup, int iters,
+                        int grid_blocks, void *stream, float *elapsed_ms);
+
+/* --------------------------------------------------------- support kernels */
+/* dst[i] = SplitMix64 counter generator word i (seeded synthetic DAG / inputs). */
+HF_API int hf_fill_splitmix64(uint64_t *dst, uint64_t nwords, uint64_t seed, void *stream);
+/* Plain device copy, the unit the HBM counters are calibrated against. */
+HF_API int hf_copy_f32(const float *src, float *dst, uint64_t n, void *stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* HFUSE_GFX950_H */

@@ -1,0 +1,210 @@
+"""GPU parity of the nonce searches, native and fused, through the C-ABI: every
+found nonce, digest and (for Ethash) mix digest must equal the CPU oracle's."""
+import numpy as np
+import pytest
+import torch
+
+from hfuse_amd import launcher as H
+from oracle import oracle as O
+
+pytestmark = pytest.mark.gpu
+
+SEED = 0x48467573
+EASY16 = (1 << 48) - 1   # 16 leading zero bits
+EASY12 = (1 << 52) - 1
+EASY10 = (1 << 54) - 1
+
+
+def sync():
+    torch.cuda.synchronize()
+
+
+def oracle_hits(found_hits):
+    found, hits = found_hits
+    return found, [(h.nonce, h.digest_bytes(), h.mix_bytes()) for h in hits]
+
+
+def test_sha256d_bitcoin_genesis_on_gpu(cuda):
+    hdr = bytes.fromhex("01000000" + "00" * 32 +
+                        "3ba3edfd7a7b12b27ac72c3e67768f617fc81bc3888a51323a9fb8aa4b1e5e4a" +
+                        "29ab5f49" + "ffff001d" + "00000000")
+    H.sha256d_set_block(hdr, 0x00000000FFFF0000)
+    res = H.new_search_results()
+    start = 2083236893 - (1 << 19)
+    H.launch_native("sha256d_gpu_hash_shared", H.sha256d_args(res, 1 << 20, start))
+    sync()
+    found, hits = H.read_search_results(res)
+    assert found == 1 and hits[0][0] == 2083236893
+    assert hits[0][1][::-1].hex() == "000000000019d6689c085ae165831e934ff763ae46a2a6c172b3f1b60a8ce26f"
+
+
+@pytest.mark.parametrize("start,count,grid,block", [(0, 1 << 20, 0, 0), (0xFFFFF000, 1 << 14, 0, 0),
+                                                    (12345, 100001, 7, 64)])
+def test_sha256d_found_set(cuda, start, count, grid, block):
+    hdr = O.seeded_bytes(80, SEED + 1)
+    H.sha256d_set_block(hdr, EASY16 if count > (1 << 17) else EASY12)
+    res = H.new_search_results()
+    H.launch_native("sha256d_gpu_hash_shared", H.sha256d_args(res, count, start), grid, block)
+    sync()
+    want = oracle_hits(O.sha256d_search(hdr, start, count, EASY16 if count > (1 << 17) else EASY12))
+    assert want[0] > 0
+    assert H.read_search_results(res) == want
+
+
+@pytest.mark.parametrize("kernel,setter,digest", [
+    ("sia_blake2b_gpu_hash", H.sia_blake2b_set_block, O.sia_blake2b_80),
+    ("blake2b_gpu_hash", H.blake2b_set_block, O.ccminer_blake2b_80)])
+def test_blake2b_found_set(cuda, kernel, setter, digest):
+    hdr = O.seeded_bytes(80, SEED + 2)
+    setter(hdr)
+    res = H.new_search_results()
+    start, count = 0xFFFF0000, 1 << 20  # wraps around 2^32 like the original's uint32 nonce
+    H.launch_native(kernel, H.blake2b_args(res, count, start, EASY16))
+    sync()
+    found, hits = H.read_search_results(res)
+    assert found > 0 and found == len(hits)
+    if kernel == "sia_blake2b_gpu_hash":
+        assert (found, hits) == oracle_hits(O.sia_search(hdr, start, count, EASY16))
+    else:
+        # brute force over the window with the oracle's single-nonce digest
+        want = []
+        for i in range(count):
+            n = (start + i) & 0xFFFFFFFF
+            d = digest(hdr, n)
+            if int.from_bytes(d[:8], "big") <= EASY16:
+                want.append((n, d, bytes(32)))
+        assert hits == sorted(want)
+
+
+def _dag(cuda, n_items, seed):
+    dag = torch.empty(n_items * 32, dtype=torch.int32, device=cuda)
+    H.fill_splitmix64(dag, seed)
+    return dag
+
+
+def test_fill_splitmix64_matches_oracle(cuda):
+    dag = _dag(cuda, 1000, SEED)
+    sync()
+    want = O.fill_splitmix64(1000 * 16, SEED).view(np.int32)
+    assert np.array_equal(dag.cpu().numpy(), want)
+
+
+@pytest.mark.parametrize("n_items", [1 << 16, 100003])  # power of two (mask) and not (modulo)
+def test_ethash_found_set(cuda, n_items):
+    dag = _dag(cuda, n_items, SEED)
+    header = O.seeded_bytes(32, SEED + 3)
+    target = (1 << 54) - 1  # 10 leading zero bits: ~64 hits in 2^16 nonces would overflow; use 2^15
+    H.ethash_set_constants(dag, n_items, header, target)
+    res = H.new_search_results()
+    start, grid = 0x0123456700000000, 256  # 256 blocks x 128 threads = 2^15 nonces
+    H.launch_native("ethash_search", H.ethash_args(res, start), grid, 128)
+    sync()
+    want = oracle_hits(O.ethash_search(None, SEED, n_items, header, start, grid * 128, target))
+    assert 0 < want[0] <= 64
+    assert H.read_search_results(res) == want
+
+
+def test_ethash_every_lane_group_position(cuda):
+    """With an all-accepting target every nonce is a hit: checks all 8 positions of a lane
+    group and all 4 interleaved hashes, mix digest and final hash, against the oracle."""
+    n_items = 4099
+    dag = _dag(cuda, n_items, SEED + 9)
+    header = O.seeded_bytes(32, SEED + 4)
+    H.ethash_set_constants(dag, n_items, header, (1 << 64) - 1)
+    res = H.new_search_results()
+    H.launch_native("ethash_search", H.ethash_args(res, 77), 1, 64)
+    sync()
+    found, hits = H.read_search_results(res)
+    assert found == 64 and [h[0] for h in hits] == list(range(77, 77 + 64))
+    for nonce, digest, mix in hits:
+        assert (mix, digest) == O.ethash_hash(None, SEED + 9, n_items, header, nonce)
+
+
+def _search_pair_args(cuda, k, count, start):
+    res = H.new_search_results()
+    if k == "sha256d_gpu_hash_shared":
+        return res, H.sha256d_args(res, count, start)
+    if k in ("sia_blake2b_gpu_hash", "blake2b_gpu_hash"):
+        return res, H.blake2b_args(res, count, start, EASY16)
+    return res, H.ethash_args(res, start)
+
+
+def test_fused_sha256d_sia(cuda, cfg):
+    h1, h2 = O.seeded_bytes(80, SEED + 5), O.seeded_bytes(80, SEED + 6)
+    H.sha256d_set_block(h1, EASY16)
+    H.sia_blake2b_set_block(h2)
+    want1 = oracle_hits(O.sha256d_search(h1, 5, 1 << 20, EASY16))
+    want2 = oracle_hits(O.sia_search(h2, 9, (1 << 20) + 333, EASY16))
+    i = cfg.find_fusion("sha256d_gpu_hash_shared", "sia_blake2b_gpu_hash")
+    for plan in (cfg.plan(i), cfg.plan(i, "hfuse", -1, 64), cfg.plan(i, "hfuse_lb", 0)):
+        r1, a1 = _search_pair_args(cuda, "sha256d_gpu_hash_shared", 1 << 20, 5)
+        r2, a2 = _search_pair_args(cuda, "sia_blake2b_gpu_hash", (1 << 20) + 333, 9)
+        plan.launch(a1, a2)
+        sync()
+        assert H.read_search_results(r1) == want1
+        assert H.read_search_results(r2) == want2
+
+
+def test_fused_ethash_sia(cuda, cfg):
+    n_items = 1 << 16
+    dag = _dag(cuda, n_items, SEED)
+    header = O.seeded_bytes(32, SEED + 7)
+    h2 = O.seeded_bytes(80, SEED + 8)
+    target = (1 << 54) - 1
+    H.ethash_set_constants(dag, n_items, header, target)
+    H.sia_blake2b_set_block(h2)
+    grid = 256
+    want1 = oracle_hits(O.ethash_search(None, SEED, n_items, header, 1000, grid * 128, target))
+    want2 = oracle_hits(O.sia_search(h2, 0, 4 * grid * 128, EASY12))
+    i = cfg.find_fusion("ethash_search", "sia_blake2b_gpu_hash")
+    j = cfg.find_fusion("sia_blake2b_gpu_hash", "ethash_search")
+    for idx, plan in ((i, cfg.plan(i)), (j, cfg.plan(j))):
+        r1 = H.new_search_results()
+        r2 = H.new_search_results()
+        a1 = H.ethash_args(r1, 1000)
+        a2 = H.blake2b_args(r2, 4 * grid * 128, 0, EASY12)
+        if idx == i:
+            plan.launch(a1, a2, grid_blocks=grid)
+        else:
+            plan.launch(a2, a1, grid_blocks=grid)
+        sync()
+        assert H.read_search_results(r1) == want1
+        assert H.read_search_results(r2) == want2
+
+
+def test_every_shipped_search_pair(cuda, cfg):
+    """All search pairs of the shipped fusion list against the natives' results."""
+    n_items = 1 << 14
+    dag = _dag(cuda, n_items, SEED)
+    header = O.seeded_bytes(32, SEED + 10)
+    hs, hb, hc = (O.seeded_bytes(80, SEED + 11 + k) for k in range(3))
+    H.ethash_set_constants(dag, n_items, header, (1 << 55) - 1)
+    H.sha256d_set_block(hs, EASY10)
+    H.sia_blake2b_set_block(hb)
+    H.blake2b_set_block(hc)
+    grid, count = 128, 128 * 128
+    names = ("ethash_search", "sha256d_gpu_hash_shared", "sia_blake2b_gpu_hash", "blake2b_gpu_hash")
+    native = {}
+    for k in names:
+        res, a = _search_pair_args(cuda, k, count, 42)
+        if k.endswith("blake2b_gpu_hash"):
+            a = H.blake2b_args(res, count, 42, EASY10)
+        H.launch_native(k, a, grid, 128)
+        sync()
+        native[k] = H.read_search_results(res)
+        assert native[k][0] > 0
+    n = 0
+    for i, (_, k1, k2) in enumerate(cfg.fusions()):
+        if k1 in names and k2 in names:
+            r1, a1 = _search_pair_args(cuda, k1, count, 42)
+            r2, a2 = _search_pair_args(cuda, k2, count, 42)
+            if k1.endswith("blake2b_gpu_hash"):
+                a1 = H.blake2b_args(r1, count, 42, EASY10)
+            if k2.endswith("blake2b_gpu_hash"):
+                a2 = H.blake2b_args(r2, count, 42, EASY10)
+            cfg.plan(i).launch(a1, a2, grid_blocks=grid)
+            sync()
+            assert H.read_search_results(r1) == native[k1], (k1, k2)
+            assert H.read_search_results(r2) == native[k2], (k1, k2)
+            n += 1
+    assert n == 7

@@ -1,0 +1,341 @@
+"""GPU parity of the five tensor kernels, native and fused, through the C-ABI.
+Bit-exact against the oracle / PyTorch CPU ops for im2col, max_pool (values and
+int64 argmax), upsample and histogram counts; 1e-5 relative for batch-norm
+mean / invstd (tolerance of the fp32 Welford tree against the fp64 two-pass)."""
+import numpy as np
+import pytest
+import torch
+
+from hfuse_amd import _lib as L
+from hfuse_amd import launcher as H
+from oracle import oracle as O
+from util import normal, pool_out, rel_err, torch_bn_stats, torch_im2col, torch_maxpool, uniform
+
+pytestmark = pytest.mark.gpu
+BN_TOL = 1e-5
+
+
+# ------------------------------------------------------------------ helpers
+class Im2col:
+    def __init__(self, dev, n, c, h, w, k=(3, 3), p=(1, 1), s=(1, 1), d=(1, 1), seed=1):
+        self.geom = (k, p, s, d)
+        self.x = uniform((n, c, h, w), seed)
+        hc = (h + 2 * p[0] - (d[0] * (k[0] - 1) + 1)) // s[0] + 1
+        wc = (w + 2 * p[1] - (d[1] * (k[1] - 1) + 1)) // s[1] + 1
+        self.xd = self.x.to(dev)
+        self.out = torch.full((n, c * k[0] * k[1], hc * wc), float("nan"), device=dev)
+        self.args = H.im2col_args(self.xd, self.out, k, p, s, d)
+
+    def check(self):
+        k, p, s, d = self.geom
+        want = torch_im2col(self.x, k, p, s, d)
+        got = self.out.cpu()
+        assert torch.equal(got, want), f"im2col mismatch: {(got != want).sum().item()} of {want.numel()}"
+        self.out.fill_(float("nan"))
+
+
+class MaxPool:
+    def __init__(self, dev, n, c, h, w, k, s, p, d=(1, 1), seed=2, x=None):
+        self.geom = (k, s, p, d)
+        self.x = uniform((n, c, h, w), seed) if x is None else x
+        ph, pw = pool_out(h, k[0], s[0], p[0], d[0]), pool_out(w, k[1], s[1], p[1], d[1])
+        self.xd = self.x.to(dev)
+        self.val = torch.full((n, c, ph, pw), float("nan"), device=dev)
+        self.idx = torch.full((n, c, ph, pw), -7, dtype=torch.int64, device=dev)
+        self.args = H.maxpool_args(self.xd, self.val, self.idx, k, s, p, d)
+
+    def check(self):
+        k, s, p, d = self.geom
+        tv, ti = torch_maxpool(self.x, k, s, p, d)
+        assert torch.equal(self.idx.cpu(), ti), "argmax mismatch"
+        assert np.array_equal(self.val.cpu().numpy(), tv.numpy(), equal_nan=True), "max value mismatch"
+        self.val.fill_(float("nan"))
+        self.idx.fill_(-7)
+
+
+class Upsample:
+    def __init__(self, dev, n, c, h, w, out_hw, seed=3):
+        self.x = uniform((n, c, h, w), seed)
+        self.out_hw = out_hw
+        self.xd = self.x.to(dev)
+        self.out = torch.full((n, c) + tuple(out_hw), float("nan"), device=dev)
+        self.args = H.upsample_nearest_args(self.xd, self.out)
+
+    def check(self):
+        want = torch.nn.functional.interpolate(self.x, size=self.out_hw, mode="nearest")
+        assert torch.equal(self.out.cpu(), want), "upsample mismatch"
+        assert np.array_equal(self.out.cpu().numpy(), O.upsample_nearest2d(self.x.numpy(), self.out_hw))
+        self.out.fill_(float("nan"))
+
+
+class BnStats:
+    def __init__(self, dev, n, c, h, w, seed=4, x=None):
+        self.x = normal((n, c, h, w), seed) if x is None else x
+        self.xd = self.x.to(dev)
+        self.mean = torch.full((c,), float("nan"), device=dev)
+        self.inv = torch.full((c,), float("nan"), device=dev)
+        self.args = H.bn_stats_args(self.xd, self.mean, self.inv, 1e-5, 0.0)
+
+    def check(self):
+        n, c = self.x.shape[:2]
+        m64, i64 = O.bn_stats_f64(self.x.reshape(n, c, -1).numpy(), 1e-5)
+        gm, gi = self.mean.cpu().numpy(), self.inv.cpu().numpy()
+        assert rel_err(gm, m64) < BN_TOL, rel_err(gm, m64)
+        assert rel_err(gi, i64) < BN_TOL, rel_err(gi, i64)
+        tm, ti = torch_bn_stats(self.x, 1e-5)
+        assert rel_err(gm, tm.numpy()) < 2 * BN_TOL and rel_err(gi, ti.numpy()) < 2 * BN_TOL
+        self.mean.fill_(float("nan"))
+        self.inv.fill_(float("nan"))
+
+
+class Histc:
+    def __init__(self, dev, n, nbins=1024, lo=0.0, hi=1.0, seed=5, x=None):
+        self.x = uniform((n,), seed, lo, hi) if x is None else x
+        self.p = (nbins, lo, hi)
+        self.xd = self.x.to(dev)
+        self.out = torch.zeros(nbins, device=dev)
+        self.args = H.histc_args(self.xd, self.out, nbins, lo, hi)
+
+    def check(self):
+        nbins, lo, hi = self.p
+        want = torch.histc(self.x, nbins, lo, hi)
+        got = self.out.cpu()
+        assert torch.equal(got, want), f"histogram mismatch in {(got != want).sum().item()} bins"
+        assert np.array_equal(got.numpy(), O.histc(self.x.numpy(), nbins, lo, hi))
+        self.out.zero_()
+
+
+def sync():
+    torch.cuda.synchronize()
+
+
+# ------------------------------------------------------------------ native kernels
+@pytest.mark.parametrize("shape", [(2, 3, 8, 8), (1, 5, 12, 20), (32, 64, 56, 56)], ids=str)
+def test_im2col_3x3(cuda, shape):
+    t = Im2col(cuda, *shape)
+    H.launch_native("im2col_kernel", t.args)
+    sync()
+    t.check()
+
+
+@pytest.mark.parametrize("case", [
+    (2, 3, 7, 9, (3, 2), (0, 1), (2, 1), (1, 1)),
+    (2, 2, 11, 10, (2, 3), (2, 2), (1, 2), (2, 1)),
+    (1, 1, 5, 5, (5, 5), (2, 2), (1, 1), (1, 1)),
+    (3, 2, 9, 10, (3, 3), (1, 1), (1, 1), (1, 1)),  # width not a multiple of 4: general path
+    (1, 2, 6, 8, (1, 1), (0, 0), (1, 1), (1, 1)),
+], ids=str)
+def test_im2col_general(cuda, case):
+    n, c, h, w, k, p, s, d = case
+    t = Im2col(cuda, n, c, h, w, k, p, s, d)
+    H.launch_native("im2col_kernel", t.args, grid_blocks=3, block_threads=64)  # forces the stride loop
+    sync()
+    t.check()
+
+
+@pytest.mark.parametrize("case", [
+    (32, 64, 112, 112, (3, 3), (2, 2), (1, 1)),   # benchmark config 1
+    (16, 128, 64, 64, (2, 2), (2, 2), (0, 0)),    # benchmark config 3
+    (2, 3, 16, 24, (3, 3), (2, 2), (1, 1)),
+    (1, 2, 8, 8, (2, 2), (2, 2), (0, 0)),
+    (2, 3, 9, 7, (2, 2), (2, 2), (0, 0)),          # odd sizes: general path
+    (2, 2, 13, 11, (3, 2), (1, 2), (1, 1)),
+    (1, 1, 6, 6, (3, 3), (1, 1), (1, 1)),
+], ids=str)
+def test_maxpool(cuda, case):
+    n, c, h, w, k, s, p = case
+    t = MaxPool(cuda, n, c, h, w, k, s, p)
+    H.launch_native("MaxPoolForward", t.args)
+    sync()
+    t.check()
+
+
+def test_maxpool_dilated(cuda):
+    t = MaxPool(cuda, 2, 2, 13, 11, (3, 2), (1, 2), (1, 1), (2, 1))
+    H.launch_native("MaxPoolForward", t.args, grid_blocks=2, block_threads=64)
+    sync()
+    t.check()
+
+
+@pytest.mark.parametrize("k,p", [((3, 3), (1, 1)), ((2, 2), (0, 0))])
+def test_maxpool_ties_nan_inf(cuda, k, p):
+    """Ties keep the first index; NaN wins; -inf planes return the first in-bounds element."""
+    x = torch.full((2, 3, 16, 16), 0.25)
+    x[0, 1] = float("-inf")
+    x[1, 0, 5, 5] = float("nan")
+    x[1, 0, 6, 6] = float("nan")
+    x[1, 1, 3, 4] = float("inf")
+    x[1, 2] = uniform((16, 16), 11).round(decimals=1)  # many exact ties
+    t = MaxPool(cuda, 2, 3, 16, 16, k, (2, 2), p, x=x)
+    H.launch_native("MaxPoolForward", t.args)
+    sync()
+    t.check()
+
+
+@pytest.mark.parametrize("shape,out", [((32, 64, 56, 56), (112, 112)), ((2, 3, 8, 12), (16, 24)),
+                                       ((2, 3, 5, 7), (10, 14)), ((1, 2, 4, 4), (7, 9)), ((1, 1, 6, 5), (3, 4))],
+                         ids=str)
+def test_upsample_nearest(cuda, shape, out):
+    t = Upsample(cuda, *shape, out)
+    H.launch_native("upsample_nearest2d_out_frame", t.args)
+    sync()
+    t.check()
+
+
+@pytest.mark.parametrize("shape", [(32, 256, 28, 28), (4, 3, 5, 10), (2, 5, 7, 1), (3, 2, 3, 3), (64, 7, 4, 4)],
+                         ids=str)
+@pytest.mark.parametrize("block", [512, 64, 1024])
+def test_bn_stats(cuda, shape, block):
+    t = BnStats(cuda, *shape)
+    H.launch_native("batch_norm_collect_statistics_kernel", t.args, block_threads=block)
+    sync()
+    t.check()
+
+
+def test_bn_stats_fewer_blocks_than_planes_and_constant_input(cuda):
+    t = BnStats(cuda, 4, 37, 6, 6)
+    H.launch_native("batch_norm_collect_statistics_kernel", t.args, grid_blocks=5, block_threads=128)
+    sync()
+    t.check()
+    c = BnStats(cuda, 4, 3, 8, 8, x=torch.full((4, 3, 8, 8), 3.5))
+    H.launch_native("batch_norm_collect_statistics_kernel", c.args)
+    sync()
+    assert torch.allclose(c.mean.cpu(), torch.full((3,), 3.5))
+    assert rel_err(c.inv.cpu().numpy(), np.full(3, 1.0 / np.sqrt(1e-5))) < BN_TOL
+
+
+def test_bn_stats_strided_input(cuda):
+    """A channel-sliced (non-contiguous) input goes down the general path."""
+    big = normal((4, 10, 6, 5), 21)
+    bd = big.to(cuda)
+    view = bd[:, 2:7]
+    mean = torch.empty(5, device=cuda)
+    inv = torch.empty(5, device=cuda)
+    a = L.BnStatsArgs()
+    a.input.data = view.data_ptr()
+    a.input.sizes[:] = [4, 5, 30]
+    a.input.strides[:] = [view.stride(0), view.stride(1), 1]
+    a.epsilon = 1e-5
+    for acc, tt in ((a.save_mean, mean), (a.save_transformed_var, inv)):
+        acc.data, acc.sizes[0], acc.strides[0] = tt.data_ptr(), 5, 1
+    H.launch_native("batch_norm_collect_statistics_kernel", a)
+    sync()
+    m64, i64 = O.bn_stats_f64(big[:, 2:7].reshape(4, 5, 30).contiguous().numpy(), 1e-5)
+    assert rel_err(mean.cpu().numpy(), m64) < BN_TOL and rel_err(inv.cpu().numpy(), i64) < BN_TOL
+
+
+@pytest.mark.parametrize("n,nbins,lo,hi", [(1 << 20, 1024, 0.0, 1.0), (100003, 1024, 0.0, 1.0), (5000, 16, 0.0, 1.0),
+                                           (70001, 256, -2.0, 2.0), (4096, 1, 0.0, 1.0), (3, 8, 0.0, 1.0)])
+def test_histc(cuda, n, nbins, lo, hi):
+    t = Histc(cuda, n, nbins, lo, hi)
+    t.x[:3] = torch.tensor([lo, hi, (lo + hi) / 2])
+    t.xd.copy_(t.x)
+    H.launch_native("kernelHistogram1D", t.args)
+    sync()
+    t.check()
+
+
+def test_histc_out_of_range_and_accumulation(cuda):
+    x = torch.tensor([-0.5, 0.0, 0.999, 1.0, 1.5, float("nan"), 0.3, 0.3])
+    t = Histc(cuda, 8, 4, 0.0, 1.0, x=x)
+    H.launch_native("kernelHistogram1D", t.args)
+    H.launch_native("kernelHistogram1D", t.args)  # counts accumulate into `a`, as in the original
+    sync()
+    assert t.out.cpu().tolist() == [2.0, 4.0, 0.0, 4.0]
+
+
+def test_histc_full_benchmark_size(cuda):
+    n = 1 << 26
+    g = torch.Generator().manual_seed(7)
+    x = torch.rand(n, generator=g, dtype=torch.float32)
+    t = Histc(cuda, n, 1024, 0.0, 1.0, x=x)
+    H.launch_native("kernelHistogram1D", t.args)
+    sync()
+    assert t.out.sum().item() == n  # every element lands in exactly one bin
+    t.check()
+
+
+# ------------------------------------------------------------------ fused pairs
+def _plans(cfg, k1, k2):
+    i = cfg.find_fusion(k1, k2)
+    plans = [("table", cfg.plan(i))]
+    for idx in range(cfg.num_splits(i)):
+        try:
+            plans.append((f"idx{idx}", cfg.plan(i, "hfuse", idx)))
+        except Exception:
+            pass
+    return plans
+
+
+def test_fused_im2col_maxpool(cuda, cfg):
+    for label, plan in _plans(cfg, "im2col_kernel", "MaxPoolForward"):
+        for a, b in ((Im2col(cuda, 32, 64, 56, 56), MaxPool(cuda, 32, 64, 112, 112, (3, 3), (2, 2), (1, 1))),
+                     (Im2col(cuda, 2, 3, 9, 10), MaxPool(cuda, 2, 3, 9, 7, (2, 2), (2, 2), (0, 0)))):
+            plan.launch(a.args, b.args)
+            sync()
+            a.check()
+            b.check()
+
+
+def test_fused_bn_upsample(cuda, cfg):
+    for label, plan in _plans(cfg, "batch_norm_collect_statistics_kernel", "upsample_nearest2d_out_frame"):
+        for a, b in ((BnStats(cuda, 32, 256, 28, 28), Upsample(cuda, 32, 64, 56, 56, (112, 112))),
+                     (BnStats(cuda, 4, 37, 6, 5), Upsample(cuda, 1, 2, 4, 4, (7, 9)))):
+            for grid in (0, 7):
+                plan.launch(a.args, b.args, grid_blocks=grid)
+                sync()
+                a.check()
+                b.check()
+
+
+def test_fused_histc_maxpool(cuda, cfg):
+    for label, plan in _plans(cfg, "kernelHistogram1D", "MaxPoolForward"):
+        for a, b in ((Histc(cuda, 1 << 22), MaxPool(cuda, 16, 128, 64, 64, (2, 2), (2, 2), (0, 0))),
+                     (Histc(cuda, 70001, 256, -2.0, 2.0), MaxPool(cuda, 2, 2, 13, 11, (3, 2), (1, 2), (1, 1)))):
+            plan.launch(a.args, b.args)
+            sync()
+            a.check()
+            b.check()
+
+
+def test_fused_barrier_modes(cuda, cfg):
+    """hist + bn both synchronise: subset counters, the shared hardware barrier and the
+    blockIdx fallback must all give the same results."""
+    i = cfg.find_fusion("kernelHistogram1D", "batch_norm_collect_statistics_kernel")
+    for mode in (L.HF_BARRIER_SUBSET, L.HF_BARRIER_MATCHED, L.HF_BARRIER_BLOCKIDX):
+        plan = cfg.plan(i)
+        plan.set_barrier_mode(mode)
+        a, b = Histc(cuda, 1 << 20), BnStats(cuda, 8, 64, 14, 14)
+        plan.launch(a.args, b.args)
+        sync()
+        a.check()
+        b.check()
+    j = cfg.find_fusion("batch_norm_collect_statistics_kernel", "upsample_nearest2d_out_frame")
+    plan = cfg.plan(j)
+    plan.set_barrier_mode(L.HF_BARRIER_BLOCKIDX)
+    a, b = BnStats(cuda, 8, 64, 14, 14), Upsample(cuda, 4, 8, 28, 28, (56, 56))
+    plan.launch(a.args, b.args)
+    sync()
+    a.check()
+    b.check()
+
+
+def test_every_shipped_tensor_pair(cuda, cfg):
+    """All tensor pairs of the shipped fusion list, small shapes, default split."""
+    makers = {
+        "im2col_kernel": lambda: Im2col(cuda, 2, 4, 12, 12),
+        "MaxPoolForward": lambda: MaxPool(cuda, 2, 4, 16, 16, (3, 3), (2, 2), (1, 1)),
+        "batch_norm_collect_statistics_kernel": lambda: BnStats(cuda, 4, 9, 6, 6),
+        "upsample_nearest2d_out_frame": lambda: Upsample(cuda, 2, 3, 8, 8, (16, 16)),
+        "kernelHistogram1D": lambda: Histc(cuda, 50000),
+    }
+    n = 0
+    for i, (_, k1, k2) in enumerate(cfg.fusions()):
+        if k1 in makers and k2 in makers:
+            a, b = makers[k1](), makers[k2]()
+            cfg.plan(i).launch(a.args, b.args)
+            sync()
+            a.check()
+            b.check()
+            n += 1
+    assert n == 10

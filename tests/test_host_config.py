@@ -1,0 +1,301 @@
+"""Host logic of the library (no GPU): YAML schemas, plans, partition parity with
+the oracle, and the error behaviour at the C-ABI."""
+import ctypes as C
+import re
+
+import pytest
+
+import hfuse_amd
+from hfuse_amd import _lib as L
+from hfuse_amd.launcher import Config
+from oracle import oracle as O
+
+KERNELS_MAP = """
+im2col_kernel:
+  KernelName: im2col_kernel
+  HasBarriers: false
+  BlockDim:
+    X: 512
+    Y: 1
+    Z: 1
+  Reg: 49
+  ExecTime: 31
+MaxPoolForward:
+  KernelName: MaxPoolForward   # trailing comment
+  HasBarriers: false
+  BlockDim:
+    X: 256
+    Y: 1
+    Z: 1
+  Reg: 24
+  ExecTime: 95
+batch_norm_collect_statistics_kernel:
+  KernelName: batch_norm_collect_statistics_kernel
+  HasBarriers: true
+  BlockDim:
+    X: 32
+    Y: 16
+    Z: 1
+  Reg: 24
+  ExecTime: 52
+"""
+
+FUSION = """
+- File: Im2ColMaxPool.cu
+  Kernels:
+   - im2col_kernel
+   - MaxPoolForward
+- File: MaxPoolBatchNorm.cu
+  Kernels:
+  - MaxPoolForward
+  - batch_norm_collect_statistics_kernel
+"""
+
+# the older per-pair form: a bare list of rows, Reg optional
+LEGACY = """
+- KernelName: im2col_kernel
+  HasBarriers: false
+  BlockDim:
+    X: 512
+    Y: 1
+    Z: 1
+- KernelName: MaxPoolForward
+  HasBarriers: false
+  BlockDim:
+    X: 256
+    Y: 1
+    Z: 1
+  Reg: 24
+"""
+
+
+def test_parse_map_form_and_fusion_list():
+    cfg = Config(FUSION, KERNELS_MAP)
+    assert cfg.num_kernels == 3 and cfg.num_fusions == 2
+    assert cfg.fusion(0) == ("Im2ColMaxPool.cu", "im2col_kernel", "MaxPoolForward")
+    assert cfg.fusion(1) == ("MaxPoolBatchNorm.cu", "MaxPoolForward", "batch_norm_collect_statistics_kernel")
+    k = cfg.kernel("batch_norm_collect_statistics_kernel")
+    assert (k.block_dim.x, k.block_dim.y, k.block_dim.z) == (32, 16, 1)
+    assert k.reg == 24 and k.exec_time == 52.0 and k.has_barriers == 1
+    assert cfg.kernel("MaxPoolForward").kernel_name == b"MaxPoolForward"
+
+
+def test_parse_legacy_list_form():
+    cfg = Config(None, LEGACY)
+    assert cfg.num_fusions == 1
+    assert cfg.fusion(0)[1:] == ("im2col_kernel", "MaxPoolForward")
+    assert cfg.kernel("im2col_kernel").reg == 0 and cfg.kernel("im2col_kernel").exec_time == -1.0
+
+
+def test_shipped_config_lists_the_five_benchmarked_pairs_first(cfg):
+    pairs = [f[1:] for f in cfg.fusions()[:5]]
+    assert pairs == [("im2col_kernel", "MaxPoolForward"),
+                     ("batch_norm_collect_statistics_kernel", "upsample_nearest2d_out_frame"),
+                     ("kernelHistogram1D", "MaxPoolForward"),
+                     ("sha256d_gpu_hash_shared", "sia_blake2b_gpu_hash"),
+                     ("ethash_search", "sia_blake2b_gpu_hash")]
+
+
+@pytest.mark.parametrize("bad,needle", [
+    ("im2col_kernel:\n  HasBarriers: false\n  BlockDim: \n    X: 1\n    Y: 1\n    Z: 1\n  Reg: 1\n", "KernelName"),
+    ("k:\n  KernelName: k\n  BlockDim:\n    X: 1\n    Y: 1\n    Z: 1\n  Reg: 1\n", "HasBarriers"),
+    ("k:\n  KernelName: k\n  HasBarriers: false\n  Reg: 1\n", "BlockDim"),
+    ("k:\n  KernelName: k\n  HasBarriers: false\n  BlockDim:\n    X: 1\n    Y: 1\n  Reg: 1\n", "BlockDim"),
+    ("k:\n  KernelName: k\n  HasBarriers: false\n  BlockDim:\n    X: 1\n    Y: 1\n    Z: 1\n", "Reg"),
+    ("k:\n  KernelName: k\n  HasBarriers: maybe\n  BlockDim:\n    X: 1\n    Y: 1\n    Z: 1\n  Reg: 1\n", "HasBarriers"),
+    ("k:\n  KernelName: k\n  HasBarriers: false\n  BlockDim:\n    X: -4\n    Y: 1\n    Z: 1\n  Reg: 1\n", "BlockDim"),
+    ("k:\n  KernelName: k\n  HasBarriers: false\n  BlockDim:\n    X: 1\n    Y: 1\n    Z: 1\n  Reg: 1\n  Bogus: 2\n", "Bogus"),
+    ("just a scalar", "expected"),
+    ("k:\n\tKernelName: k\n", "tab"),
+    ("", "expected"),
+])
+def test_kernel_table_schema_errors(bad, needle):
+    with pytest.raises(hfuse_amd.HfuseError) as e:
+        Config("- File: f\n  Kernels:\n    - k\n    - k\n", bad)
+    assert e.value.code == L.HF_EPARSE and needle in e.value.message
+
+
+def test_fusion_list_errors():
+    with pytest.raises(hfuse_amd.HfuseError) as e:
+        Config("- File: f\n  Kernels:\n    - im2col_kernel\n    - nope\n", KERNELS_MAP)
+    assert e.value.code == L.HF_EPARSE and "nope" in e.value.message
+    with pytest.raises(hfuse_amd.HfuseError) as e:
+        Config("- File: f\n  Kernels:\n    - im2col_kernel\n", KERNELS_MAP)
+    assert "exactly two" in e.value.message
+    with pytest.raises(hfuse_amd.HfuseError) as e:
+        Config("- Kernels:\n    - im2col_kernel\n    - MaxPoolForward\n", KERNELS_MAP)
+    assert "File" in e.value.message
+    with pytest.raises(hfuse_amd.HfuseError) as e:
+        Config.from_files("/nonexistent/fusion.yaml", "/nonexistent/kernels.yaml")
+    assert e.value.code == L.HF_EIO and "failed to read configs" in e.value.message
+
+
+def _rows(cfg, i):
+    _, k1, k2 = cfg.fusion(i)
+    out = []
+    for k in (k1, k2):
+        r = cfg.kernel(k)
+        out.append(((r.block_dim.x, r.block_dim.y, r.block_dim.z), r.reg, r.exec_time))
+    return out
+
+
+def test_partition_matches_oracle_for_every_shipped_pair_and_split(cfg):
+    """Product partition == oracle Context with the wavefront granule and gfx950 register file."""
+    checked = 0
+    for i in range(cfg.num_fusions):
+        rows = _rows(cfg, i)
+        total = sum(r[0][0] * r[0][1] * r[0][2] for r in rows)
+        assert cfg.num_splits(i) == len(O.enumerate_splits(rows, granule=64))
+        for idx in range(cfg.num_splits(i)):
+            split = 128 * (idx + 1)
+            ex = [(rows[0][0], rows[0][1], float(split)), (rows[1][0], rows[1][1], float(total - split))]
+            for preset, lb in (("hfuse", False), ("hfuse_lb", True)):
+                want = O.context(ex, launch_bound=lb, imbalanced=True, granule=64, reg_file=4 * 512 * 64,
+                                 max_threads=2048)
+                try:
+                    plan = cfg.plan(i, preset, idx)
+                except hfuse_amd.HfuseError as e:
+                    # legal in the reference's arithmetic, refused here: part not a multiple of 64 / Y
+                    assert e.code == L.HF_EINVAL
+                    continue
+                got = plan.partition
+                assert list(got.lo) == list(want.lo) and list(got.hi) == list(want.hi)
+                for h in range(2):
+                    assert (got.block_dim[h].x, got.block_dim[h].y) == (want.block_dim[h].x, want.block_dim[h].y)
+                assert got.launch_threads == want.launch_threads and got.launch_blocks == want.launch_blocks
+                assert got.name.decode().endswith(f"_fused_kernel_{preset}_idx_{idx}")
+                checked += 1
+    assert checked > 40
+
+
+def test_fused_name_and_presets():
+    cfg = Config(FUSION, KERNELS_MAP)
+    p = cfg.plan(0, "hfuse", 1)
+    assert p.name == "im2col_kernel_MaxPoolForward_fused_kernel_hfuse_idx_1"
+    assert list(p.partition.hi) == [256, 768]
+    v = cfg.plan(0, "vfuse_lb", 0).partition
+    assert v.name == b"im2col_kernel_MaxPoolForward_fused_kernel_vfuse_lb_idx_0"
+    assert (list(v.lo), list(v.hi), v.launch_threads) == ([0, 0], [512, 256], 512)
+    with pytest.raises(hfuse_amd.HfuseError) as e:
+        cfg.plan(0, "hfuse_bar_sync", 0)
+    assert e.value.code == L.HF_ENOTFOUND
+    # ExecTime-proportional split (KernelFusion.h:63-72) at the wavefront granule:
+    # int(31/126 * 768 / 64) * 64 = 128
+    assert list(cfg.plan(0, "hfuse", L.HF_SPLIT_EXECTIME).partition.hi) == [128, 768]
+
+
+def test_split_rules():
+    cfg = Config(FUSION, KERNELS_MAP)
+    with pytest.raises(hfuse_amd.HfuseError):
+        cfg.plan(0, "hfuse", 5)  # 768 threads: indices 0..4 only
+    with pytest.raises(hfuse_amd.HfuseError) as e:
+        cfg.plan(0, "hfuse", L.HF_SPLIT_TABLE, 100)
+    assert "multiple" in e.value.message
+    with pytest.raises(hfuse_amd.HfuseError):
+        cfg.plan(0, "hfuse", L.HF_SPLIT_TABLE, 768)  # nothing left for kernel 2
+    p = cfg.plan(1, "hfuse", L.HF_SPLIT_TABLE, 256).partition  # bn keeps Y = 16 -> X = 32
+    assert (p.block_dim[1].x, p.block_dim[1].y, p.hi[1]) == (32, 16, 768)
+    p = cfg.plan(1, "hfuse", L.HF_SPLIT_TABLE, 448).partition  # 320 threads left = 20 x 16, five waves
+    assert (p.block_dim[1].x, p.block_dim[1].y) == (20, 16)
+    big = KERNELS_MAP.replace("X: 512", "X: 1024")
+    with pytest.raises(hfuse_amd.HfuseError) as e:
+        Config(FUSION, big).plan(0, "hfuse")
+    assert "1024" in e.value.message
+
+
+def test_local_index_follows_the_remap(cfg):
+    plan = cfg.plan(cfg.find_fusion("upsample_nearest2d_out_frame", "batch_norm_collect_statistics_kernel"))
+    part = plan.partition
+    dim = (part.block_dim[1].x, part.block_dim[1].y, part.block_dim[1].z)
+    for tid in (part.lo[1], part.lo[1] + 65, part.hi[1] - 1):
+        assert plan.local_index(1, tid) == O.remap_tid(tid, part.lo[1], dim)
+    with pytest.raises(hfuse_amd.HfuseError):
+        plan.local_index(1, part.lo[1] - 1)
+
+
+def test_barrier_policy(cfg):
+    assert cfg.plan(0).partition.barrier_mode == L.HF_BARRIER_NONE
+    bn_up = cfg.plan(1)
+    assert bn_up.partition.barrier_mode == L.HF_BARRIER_SUBSET
+    with pytest.raises(hfuse_amd.HfuseError):
+        bn_up.set_barrier_mode(L.HF_BARRIER_MATCHED)  # upsample never synchronises
+    with pytest.raises(hfuse_amd.HfuseError):
+        bn_up.set_barrier_mode(L.HF_BARRIER_NONE)
+    bn_up.set_barrier_mode(L.HF_BARRIER_BLOCKIDX)
+    both = cfg.plan(cfg.find_fusion("kernelHistogram1D", "batch_norm_collect_statistics_kernel"))
+    both.set_barrier_mode(L.HF_BARRIER_MATCHED)
+    assert both.partition.barrier_mode == L.HF_BARRIER_MATCHED
+
+
+def test_unknown_and_unbuilt_kernels():
+    table = KERNELS_MAP + """
+upsample_bilinear2d_out_frame:
+  KernelName: upsample_bilinear2d_out_frame
+  HasBarriers: false
+  BlockDim:
+    X: 512
+    Y: 1
+    Z: 1
+  Reg: 43
+foo:
+  KernelName: foo
+  HasBarriers: false
+  BlockDim:
+    X: 256
+    Y: 1
+    Z: 1
+  Reg: 8
+"""
+    fusion = ("- File: a\n  Kernels:\n    - MaxPoolForward\n    - upsample_bilinear2d_out_frame\n"
+              "- File: b\n  Kernels:\n    - foo\n    - MaxPoolForward\n")
+    cfg = Config(fusion, table)
+    with pytest.raises(hfuse_amd.HfuseError) as e:
+        cfg.plan(0)
+    assert e.value.code == L.HF_EUNSUPPORTED
+    with pytest.raises(hfuse_amd.HfuseError) as e:
+        cfg.plan(1)
+    assert e.value.code == L.HF_ENOTFOUND
+
+
+def test_launch_argument_errors_never_reach_the_gpu(cfg):
+    """Null pointers and inconsistent shapes are refused on the host."""
+    lib = L.lib()
+    plan = cfg.plan(0)
+    a, b = L.Im2colArgs(), L.MaxPoolArgs()
+    assert lib.hf_launch_fused(plan._h, C.byref(a), C.byref(b), 0, None) == L.HF_EINVAL
+    assert b"null data pointer" in lib.hf_last_error()
+    assert lib.hf_launch_fused(plan._h, None, C.byref(b), 0, None) == L.HF_EINVAL
+    assert lib.hf_launch_native(b"no_such_kernel", C.byref(a), 0, 0, None) == L.HF_ENOTFOUND
+    assert lib.hf_launch_native(None, C.byref(a), 0, 0, None) == L.HF_EINVAL
+    a.data_im = a.data_col = 256
+    a.n, a.height, a.width, a.kernel_h, a.kernel_w = 64, 8, 8, 3, 3
+    a.stride_h = a.stride_w = a.dilation_h = a.dilation_w = 1
+    a.pad_h = a.pad_w = 1
+    a.height_col, a.width_col = 8, 7  # does not follow from the geometry
+    assert lib.hf_launch_native(b"im2col_kernel", C.byref(a), 0, 0, None) == L.HF_EINVAL
+    assert b"height_col" in lib.hf_last_error()
+    e = L.EthashArgs()
+    e.g_output = 256
+    assert lib.hf_launch_native(b"ethash_search", C.byref(e), 0, 0, None) == L.HF_EINVAL
+    assert b"hf_ethash_set_constants" in lib.hf_last_error()
+    h = L.HistcArgs()
+    h.a.data = h.b.data = 256
+    h.a.dims = h.b.dims = 1
+    h.nbins, h.minvalue, h.maxvalue = 8, 1.0, 0.0
+    assert lib.hf_launch_native(b"kernelHistogram1D", C.byref(h), 0, 0, None) == L.HF_EINVAL
+    assert b"max must be larger than min" in lib.hf_last_error()
+    v = cfg.plan(0, "vfuse")
+    assert lib.hf_launch_fused(v._h, C.byref(a), C.byref(b), 0, None) in (L.HF_EINVAL, L.HF_EUNSUPPORTED)
+
+
+def test_header_symbols_are_all_exported():
+    """Every function include/hfuse_gfx950.h declares is exported by the built library."""
+    import os
+    hdr = open(os.path.join(os.path.dirname(hfuse_amd.__file__), "..", "include", "hfuse_gfx950.h")).read()
+    declared = set(re.findall(r"HF_API\s+[\w\s\*]+?\b(hf_\w+)\s*\(", hdr))
+    assert len(declared) >= 20
+    assert declared == set(L.PROTOTYPES), declared ^ set(L.PROTOTYPES)
+    lib = L.lib()
+    for name in declared:
+        assert hasattr(lib, name), name
+    assert lib.hf_version() >= 100
