@@ -1,0 +1,440 @@
+#!/usr/bin/env python3
+"""Benchmark of the five horizontally fused pairs on one MI355X.
+
+A "step" is one launch of the fused kernel of the headline pair (batch-norm
+collect-statistics + upsample_nearest2d at its full shape) over one set of
+synthetic inputs already resident in HBM.  For every pair the script also times
+the two native kernels alone and back to back on one stream, so the metric of
+the reference (fused time vs. the two native launches) can be read per pair.
+
+Prints ONE JSON line.  `value` is the headline pair's speedup in percent,
+(t_back_to_back / t_fused - 1) * 100; `pairs` carries the same plus absolute
+GB/s or MH/s and roofline fractions for all five pairs; `roofline` is the
+headline pair's fused kernel against HBM peak; `cpu_baseline` is the CPU oracle
+timed on this host's cores on a bounded sample.
+"""
+from __future__ import annotations
+
+import argparse
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+HBM_PEAK_GBPS = 8000.0            # MI355X HBM3E
+VALU_PEAK_GOPS = 256 * 64 * 2.4   # 256 CUs x 64 lanes x 2.4 GHz int32 op/s, in Gop/s
+SEED = 0x48467573
+
+# textbook primitive-op counts per hash (add / logic / rotate / shift = 1 each)
+OPS_SHA256D = 4336
+OPS_BLAKE2B = 2528
+ETHASH_BYTES = 8192               # 64 accesses x 128 bytes of DAG per hash
+
+
+def parse():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=200)
+    ap.add_argument("--warmup", type=int, default=20)
+    ap.add_argument("--pairs", default="all", help="comma list of pair names, or 'all'")
+    ap.add_argument("--headline", default="bn_upsample")
+    ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    ap.add_argument("--no-sweep", action="store_true", help="time the table split only")
+    ap.add_argument("--fused-only", action="store_true", help="launch only the fused kernel (profiling runs)")
+    ap.add_argument("--search-log2", type=int, default=None, help="override log2 of the nonce ranges (debug)")
+    return ap.parse_args()
+
+
+# ------------------------------------------------------------------ workloads
+class TensorPair:
+    """One tensor pair: `nsets` independent input/output sets so repeats miss the last-level cache."""
+
+    def __init__(self, name, k1, k2, make_set, bytes1, bytes2, min_footprint=1 << 30):
+        self.name, self.k1, self.k2 = name, k1, k2
+        self.bytes1, self.bytes2 = bytes1, bytes2
+        self.sets = []
+        footprint = 0
+        while footprint < min_footprint or len(self.sets) < 2:
+            s = make_set(len(self.sets))
+            self.sets.append(s)
+            footprint += s["footprint"]
+        self.args1 = [s["a1"] for s in self.sets]
+        self.args2 = [s["a2"] for s in self.sets]
+
+
+def rand(shape, seed, lo=-1.0, hi=1.0, dev="cuda"):
+    import torch
+    g = torch.Generator(device=dev).manual_seed(seed)
+    return torch.rand(shape, generator=g, device=dev, dtype=torch.float32) * (hi - lo) + lo
+
+
+def randn(shape, seed, mean, std, dev="cuda"):
+    import torch
+    g = torch.Generator(device=dev).manual_seed(seed)
+    return torch.randn(shape, generator=g, device=dev, dtype=torch.float32) * std + mean
+
+
+def build_tensor_pairs(names):
+    import torch
+    from hfuse_amd import launcher as H
+    pairs = {}
+
+    def nbytes(*ts):
+        return sum(t.numel() * t.element_size() for t in ts)
+
+    if "im2col_maxpool" in names:
+        def mk(i):
+            x = rand((32, 64, 56, 56), SEED + 10 * i)
+            col = torch.empty((32, 576, 3136), device="cuda")
+            y = rand((32, 64, 112, 112), SEED + 10 * i + 1)
+            val = torch.empty((32, 64, 56, 56), device="cuda")
+            idx = torch.empty((32, 64, 56, 56), dtype=torch.int64, device="cuda")
+            return dict(keep=(x, col, y, val, idx), footprint=nbytes(x, col, y, val, idx),
+                        a1=H.im2col_args(x, col), a2=H.maxpool_args(y, val, idx, (3, 3), (2, 2), (1, 1)))
+        pairs["im2col_maxpool"] = TensorPair("im2col_maxpool", "im2col_kernel", "MaxPoolForward", mk,
+                                             256901120, 179830784)
+    if "bn_upsample" in names:
+        def mk(i):
+            x = randn((32, 256, 28, 28), SEED + 10 * i + 2, 0.5, 2.0)
+            mean = torch.empty(256, device="cuda")
+            inv = torch.empty(256, device="cuda")
+            u = rand((32, 64, 56, 56), SEED + 10 * i + 3)
+            out = torch.empty((32, 64, 112, 112), device="cuda")
+            return dict(keep=(x, mean, inv, u, out), footprint=nbytes(x, u, out),
+                        a1=H.bn_stats_args(x, mean, inv, 1e-5, 0.0), a2=H.upsample_nearest_args(u, out))
+        pairs["bn_upsample"] = TensorPair("bn_upsample", "batch_norm_collect_statistics_kernel",
+                                          "upsample_nearest2d_out_frame", mk, 25692160, 128450560)
+    if "histc_maxpool" in names:
+        def mk(i):
+            x = rand((1 << 26,), SEED + 10 * i + 4, 0.0, 1.0)
+            hist = torch.zeros(1024, device="cuda")
+            y = rand((16, 128, 64, 64), SEED + 10 * i + 5)
+            val = torch.empty((16, 128, 32, 32), device="cuda")
+            idx = torch.empty((16, 128, 32, 32), dtype=torch.int64, device="cuda")
+            return dict(keep=(x, hist, y, val, idx), footprint=nbytes(x, y, val, idx),
+                        a1=H.histc_args(x, hist, 1024, 0.0, 1.0), a2=H.maxpool_args(y, val, idx, (2, 2), (2, 2), (0, 0)))
+        pairs["histc_maxpool"] = TensorPair("histc_maxpool", "kernelHistogram1D", "MaxPoolForward", mk,
+                                            268439552, 58720256)
+    return pairs
+
+
+def candidate_plans(cfg, k1, k2, sweep):
+    i = cfg.find_fusion(k1, k2)
+    out = [("table", cfg.plan(i))]
+    if sweep:
+        for idx in range(cfg.num_splits(i)):
+            try:
+                out.append((f"idx_{idx}", cfg.plan(i, "hfuse", idx)))
+            except Exception:
+                pass
+    return out
+
+
+def time_tensor_pair(cfg, pair, steps, warmup, sweep, fused_only):
+    """-> dict with per-launch milliseconds of native A, native B, back-to-back and the best fused split."""
+    plans = candidate_plans(cfg, pair.k1, pair.k2, sweep)
+    base = plans[0][1]
+    res = {}
+    if not fused_only:
+        res["t_a_ms"] = base.time(0, pair.args1, pair.args2, warmup, steps) / steps
+        res["t_b_ms"] = base.time(1, pair.args1, pair.args2, warmup, steps) / steps
+        res["t_b2b_ms"] = base.time(2, pair.args1, pair.args2, warmup, steps) / steps
+    best = None
+    probe = max(20, steps // 4)
+    for label, plan in plans:
+        t = plan.time(3, pair.args1, pair.args2, max(5, warmup // 2), probe) / probe
+        if best is None or t < best[0]:
+            best = (t, label, plan)
+    _, label, plan = best
+    res["t_fused_ms"] = plan.time(3, pair.args1, pair.args2, warmup, steps) / steps
+    res["split"] = label
+    part = plan.partition
+    res["fused_name"] = part.name.decode()
+    res["threads"] = [part.hi[0] - part.lo[0], part.hi[1] - part.lo[1]]
+    res["plan"] = plan
+    return res
+
+
+# ------------------------------------------------------------------ searches
+def time_events(fn, iters):
+    import torch
+    a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    torch.cuda.synchronize()
+    a.record()
+    for _ in range(iters):
+        fn()
+    b.record()
+    b.synchronize()
+    return a.elapsed_time(b) / iters
+
+
+def run_search_pair(cfg, name, log2_a, log2_b, sweep, fused_only, iters=2):
+    """sha256d+blake2b (log2 nonces each) or ethash+blake2b."""
+    import torch
+    from hfuse_amd import launcher as H
+    from oracle import oracle as O
+    ethash = name == "ethash_blake2b"
+    k1 = "ethash_search" if ethash else "sha256d_gpu_hash_shared"
+    k2 = "sia_blake2b_gpu_hash"
+    na, nb = 1 << log2_a, 1 << log2_b
+    target32 = (1 << 32) - 1            # 32 leading zero bits
+    hdr_a = O.seeded_bytes(32 if ethash else 80, SEED + 100)
+    hdr_b = O.seeded_bytes(80, SEED + 101)
+    H.sia_blake2b_set_block(hdr_b)
+    keep = []
+    if ethash:
+        n_items = 1 << 25               # 4 GiB of 128-byte items
+        dag = torch.empty(n_items * 32, dtype=torch.int32, device="cuda")
+        H.fill_splitmix64(dag, SEED)
+        torch.cuda.synchronize()
+        eth_target = (1 << 40) - 1      # 24 leading zero bits: ~16 expected hits in 2^28 nonces
+        H.ethash_set_constants(dag, n_items, hdr_a, eth_target)
+        keep.append(dag)
+    else:
+        H.sha256d_set_block(hdr_a, target32)
+
+    def fresh():
+        ra, rb = H.new_search_results(), H.new_search_results()
+        a1 = H.ethash_args(ra, 0) if ethash else H.sha256d_args(ra, na, 0)
+        a2 = H.blake2b_args(rb, nb, 0, target32)
+        return ra, rb, a1, a2
+
+    grid = na // 128 if ethash else 0
+    ra, rb, a1, a2 = fresh()
+    res = {}
+    plans = candidate_plans(cfg, k1, k2, sweep)
+    base = plans[0][1]
+    if not fused_only:
+        res["t_a_ms"] = base.time(0, [a1], [a2], 1, iters, grid) / iters
+        res["t_b_ms"] = base.time(1, [a1], [a2], 1, iters, 0) / iters
+        res["t_b2b_ms"] = base.time(2, [a1], [a2], 0, iters, grid) / iters
+    best = None
+    for label, plan in plans:
+        t = plan.time(3, [a1], [a2], 0, 1, grid)
+        if best is None or t < best[0]:
+            best = (t, label, plan)
+    _, label, plan = best
+    res["t_fused_ms"] = plan.time(3, [a1], [a2], 0, iters, grid) / iters
+    res["split"] = label
+    part = plan.partition
+    res["fused_name"] = part.name.decode()
+    res["threads"] = [part.hi[0] - part.lo[0], part.hi[1] - part.lo[1]]
+    # Correctness of what was just timed: one more fused pass into fresh buffers, every hit
+    # re-hashed by the oracle, and the found sets compared with the native kernels' found sets.
+    fa, fb, f1, f2 = fresh()
+    plan.launch(f1, f2, grid_blocks=grid)
+    na_, nb_, n1, n2 = fresh()
+    H.launch_native(k1, n1, grid, 128)
+    H.launch_native(k2, n2, 0, 128)
+    torch.cuda.synchronize()
+    got_a, got_b = H.read_search_results(fa), H.read_search_results(fb)
+    assert got_a == H.read_search_results(na_) and got_b == H.read_search_results(nb_), "fused and native found sets differ"
+    for nonce, digest, mix in got_a[1]:
+        if ethash:
+            assert (mix, digest) == O.ethash_hash(None, SEED, 1 << 25, hdr_a, nonce), "ethash hit differs from the oracle"
+        else:
+            assert digest == O.sha256d_80(hdr_a, nonce), "sha256d hit differs from the oracle"
+    for nonce, digest, _ in got_b[1]:
+        assert digest == O.sia_blake2b_80(hdr_b, nonce & 0xFFFFFFFF), "blake2b hit differs from the oracle"
+    res["hits"] = [got_a[0], got_b[0]]
+    res["nonces"] = [na, nb]
+    del keep
+    return res
+
+
+# ------------------------------------------------------------------ CPU baseline
+def cpu_baseline_tensor(name, budget_s=12.0):
+    """Oracle (C port, OpenMP) and PyTorch CPU ops on the full shape of the pair, repeated within a budget."""
+    import torch
+    from oracle import oracle as O
+    import numpy as np
+    g = torch.Generator().manual_seed(1)
+    if name == "bn_upsample":
+        x = (torch.randn((32, 256, 28, 28), generator=g) * 2 + 0.5).contiguous()
+        u = torch.rand((32, 64, 56, 56), generator=g).contiguous()
+        xn, un = x.reshape(32, 256, 784).numpy(), u.numpy()
+        port = lambda: (O.bn_stats(xn, 1e-5), O.upsample_nearest2d(un, (112, 112)))
+        ref = lambda: (torch.native_batch_norm(x, None, None, None, None, True, 0.0, 1e-5),
+                       torch.nn.functional.interpolate(u, scale_factor=2, mode="nearest"))
+        nbytes = 25692160 + 128450560
+    elif name == "im2col_maxpool":
+        x = torch.rand((32, 64, 56, 56), generator=g).contiguous()
+        y = torch.rand((32, 64, 112, 112), generator=g).contiguous()
+        xn, yn = x.reshape(2048, 56, 56).numpy(), y.numpy()
+        port = lambda: (O.im2col(xn, (3, 3), (1, 1), (1, 1)), O.max_pool(yn, (3, 3), (2, 2), (1, 1)))
+        ref = lambda: (torch.nn.functional.unfold(x, 3, padding=1), torch.nn.functional.max_pool2d(y, 3, 2, 1, return_indices=True))
+        nbytes = 256901120 + 179830784
+    else:
+        x = torch.rand((1 << 26,), generator=g)
+        y = torch.rand((16, 128, 64, 64), generator=g).contiguous()
+        xn, yn = x.numpy(), y.numpy()
+        port = lambda: (O.histc(xn, 1024, 0.0, 1.0), O.max_pool(yn, (2, 2), (2, 2), (0, 0)))
+        ref = lambda: (torch.histc(x, 1024, 0, 1), torch.nn.functional.max_pool2d(y, 2, 2, 0, return_indices=True))
+        nbytes = 268439552 + 58720256
+
+    def clock(fn):
+        fn()
+        t0, n = time.perf_counter(), 0
+        while n < 2 or time.perf_counter() - t0 < budget_s / 2:
+            fn()
+            n += 1
+        return (time.perf_counter() - t0) / n, n
+    tp, npass = clock(port)
+    tr, nref = clock(ref)
+    return dict(port_ms=tp * 1e3, port_gbps=nbytes / tp / 1e9, port_passes=npass,
+                torch_cpu_ms=tr * 1e3, torch_cpu_gbps=nbytes / tr / 1e9, torch_threads=torch.get_num_threads(),
+                threads=O.num_threads())
+
+
+def cpu_baseline_search(name, seconds=6.0):
+    from oracle import oracle as O
+    hdr80 = O.seeded_bytes(80, SEED + 101)
+    out = {"threads": O.num_threads()}
+
+    def rate(fn, n0):
+        n = n0
+        while True:
+            t0 = time.perf_counter()
+            fn(n)
+            dt = time.perf_counter() - t0
+            if dt > seconds / 3 or n >= 1 << 28:
+                return n / dt / 1e6, n
+            n *= 4
+    out["blake2b_mhs"], out["blake2b_sample"] = rate(lambda n: O.sia_search(hdr80, 0, n, 0), 1 << 18)
+    if name == "sha256d_blake2b":
+        out["sha256d_mhs"], out["sha256d_sample"] = rate(lambda n: O.sha256d_search(hdr80, 0, n, 0), 1 << 18)
+    else:
+        hdr32 = O.seeded_bytes(32, SEED + 100)
+        # the same 4 GiB synthetic DAG, evaluated on the fly by the counter generator
+        out["ethash_mhs"], out["ethash_sample"] = rate(
+            lambda n: O.ethash_search(None, SEED, 1 << 25, hdr32, 0, n, 0), 1 << 12)
+    return out
+
+
+# ------------------------------------------------------------------ main
+def main():
+    args = parse()
+    if args.gpus != 1:
+        print("bench.py: this build runs on one GPU (every pair shards without exchange; see DESIGN.md); "
+              "--gpus must be 1", file=sys.stderr)
+        sys.exit(2)
+    import torch
+    import hfuse_amd
+    assert torch.cuda.is_available(), "bench.py needs an MI355X"
+    hfuse_amd._lib.lib()  # fail loudly if the HIP library is missing
+    torch.cuda.set_device(0)
+    cfg = hfuse_amd.default_config()
+    all_names = ["im2col_maxpool", "bn_upsample", "histc_maxpool", "sha256d_blake2b", "ethash_blake2b"]
+    names = all_names if args.pairs == "all" else [n for n in args.pairs.split(",") if n]
+    if args.headline not in names:
+        names.append(args.headline)
+    sweep = not args.no_sweep
+    report = {}
+
+    # tensor pairs one at a time (each holds ~1 GiB of rotating buffers)
+    headline = None
+    for name in [n for n in names if n in ("im2col_maxpool", "bn_upsample", "histc_maxpool")]:
+        pair = build_tensor_pairs([name])[name]
+        torch.cuda.synchronize()
+        r = time_tensor_pair(cfg, pair, args.steps, args.warmup, sweep, args.fused_only)
+        plan = r.pop("plan")
+        total = pair.bytes1 + pair.bytes2
+        r["bytes"] = [pair.bytes1, pair.bytes2]
+        r["fused_gbps"] = total / (r["t_fused_ms"] * 1e-3) / 1e9
+        r["roofline_frac"] = r["fused_gbps"] / HBM_PEAK_GBPS
+        if not args.fused_only:
+            r["a_gbps"] = pair.bytes1 / (r["t_a_ms"] * 1e-3) / 1e9
+            r["b_gbps"] = pair.bytes2 / (r["t_b_ms"] * 1e-3) / 1e9
+            r["speedup_pct"] = (r["t_b2b_ms"] / r["t_fused_ms"] - 1.0) * 100.0
+        if name == args.headline:
+            # the timed region of the contract: exactly K steps between two synchronisations
+            plan.time(3, pair.args1, pair.args2, args.warmup, 1)
+            torch.cuda.synchronize()
+            t0 = time.perf_counter()
+            ev_ms = plan.time(3, pair.args1, pair.args2, 0, args.steps)
+            torch.cuda.synchronize()
+            wall_ms = (time.perf_counter() - t0) * 1e3
+            headline = dict(r, wall_ms_per_step=wall_ms / args.steps, event_ms_per_step=ev_ms / args.steps,
+                            total_bytes=total, nsets=len(pair.sets))
+        report[name] = r
+        del pair, plan
+        torch.cuda.empty_cache()
+
+    for name in [n for n in names if n in ("sha256d_blake2b", "ethash_blake2b")]:
+        la = args.search_log2 or (28 if name == "ethash_blake2b" else 30)
+        lb = args.search_log2 + 2 if (args.search_log2 and name == "ethash_blake2b") else (args.search_log2 or 30)
+        r = run_search_pair(cfg, name, la, lb, sweep, args.fused_only)
+        na, nb = r["nonces"]
+        tf = r["t_fused_ms"] * 1e-3
+        r["fused_mhs"] = [na / tf / 1e6, nb / tf / 1e6]
+        if name == "sha256d_blake2b":
+            ops = na * OPS_SHA256D + nb * OPS_BLAKE2B
+            r["fused_valu_gops"] = ops / tf / 1e9
+            r["roofline_frac"] = r["fused_valu_gops"] / VALU_PEAK_GOPS
+            r["roofline_bound"] = "valu_int32"
+        else:
+            r["dag_gbps"] = na * ETHASH_BYTES / tf / 1e9
+            r["roofline_frac"] = r["dag_gbps"] / HBM_PEAK_GBPS
+            r["roofline_bound"] = "hbm"
+            r["blake2b_valu_frac"] = nb * OPS_BLAKE2B / tf / 1e9 / VALU_PEAK_GOPS
+        if not args.fused_only:
+            r["a_mhs"] = na / (r["t_a_ms"] * 1e-3) / 1e6
+            r["b_mhs"] = nb / (r["t_b_ms"] * 1e-3) / 1e6
+            r["speedup_pct"] = (r["t_b2b_ms"] / r["t_fused_ms"] - 1.0) * 100.0
+        report[name] = r
+        torch.cuda.empty_cache()
+
+    cpu = None
+    if not args.no_cpu:
+        from oracle import oracle as O
+        for name in names:
+            if name in ("sha256d_blake2b", "ethash_blake2b"):
+                report[name]["cpu"] = cpu_baseline_search(name)
+            elif name != args.headline:
+                report[name]["cpu"] = cpu_baseline_tensor(name, 8.0)
+        c = cpu_baseline_tensor(args.headline, 16.0)
+        report[args.headline]["cpu"] = c
+        cpu = {"value": c["port_gbps"], "unit": "GB/s", "cores": c["threads"], "kind": "port",
+               "sample": f"{c['port_passes']} full passes of the headline pair's CPU port (oracle, OpenMP) "
+                         f"at {c['port_ms']:.1f} ms each; PyTorch CPU ops on the same tensors: "
+                         f"{c['torch_cpu_gbps']:.2f} GB/s on {c['torch_threads']} threads",
+               "host_cpus": os.cpu_count()}
+
+    h = headline or {}
+    n_fast = sum(1 for r in report.values() if r.get("speedup_pct", -1e9) >= 10.0)
+    line = {
+        "metric": "fused-pair time vs back-to-back launches (speedup %)",
+        "value": h.get("speedup_pct"),
+        "unit": "%",
+        "n_gpus": 1,
+        "steps": args.steps,
+        "warmup": args.warmup,
+        "ms_per_step": h.get("wall_ms_per_step"),
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": "f32",
+        "data": "synthetic (seeded), inputs resident in HBM, rotating buffer sets",
+        "config": {"workload": "configs[1]: batch_norm_collect_statistics [32,256,28,28] + upsample_nearest2d "
+                               "[32,64,56,56]->[32,64,112,112], one fused launch per step",
+                   "fused_kernel": h.get("fused_name"), "split_threads": h.get("threads"),
+                   "buffer_sets": h.get("nsets")},
+        "throughput": {"value": h.get("fused_gbps"), "unit": "GB/s (algorithmic bytes of both kernels / fused time)"},
+        "pairs_at_least_10pct_faster": n_fast,
+        "roofline": {"bound": "hbm", "achieved": (h["total_bytes"] / (h["event_ms_per_step"] * 1e-3) / 1e9) if h else None,
+                     "peak": HBM_PEAK_GBPS, "unit": "GB/s",
+                     "frac": (h["total_bytes"] / (h["event_ms_per_step"] * 1e-3) / 1e9 / HBM_PEAK_GBPS) if h else None,
+                     "traffic": None,
+                     "kernel": h.get("fused_name"), "algorithmic_bytes_per_launch": h.get("total_bytes"),
+                     "avg_launch_ms": h.get("event_ms_per_step")},
+        "cpu_baseline": cpu,
+        "pairs": report,
+    }
+    print(json.dumps(line))
+
+
+if __name__ == "__main__":
+    main()

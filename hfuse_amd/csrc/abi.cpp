@@ -140,12 +140,17 @@ int cu_count() {
 // ------------------------------------------------------- argument validation
 struct Prepared {
   KernelId id = K_COUNT;
-  alignas(16) unsigned char blob[320];  // device-side argument struct
+  alignas(16) unsigned char blob[512];  // device-side argument struct
   unsigned hint = 0;
   unsigned lds = 0;
   bool exact_grid = false;  // the grid decides the amount of work (ethash)
   unsigned long long items = 0;  // work items of one pass at the chosen hint
 };
+
+static_assert(sizeof(hf_im2col_args) <= 512 && sizeof(hf_maxpool_args) <= 512 && sizeof(hf_bn_stats_args) <= 512 &&
+                  sizeof(hf_upsample_nearest_args) <= 512 && sizeof(hf_histc_args) <= 512 &&
+                  sizeof(EthashDevArgs) <= 512 && sizeof(Sha256dDevArgs) <= 512 && sizeof(Blake2bDevArgs) <= 512,
+              "argument blob too small");
 
 bool aligned16(const void *p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
 
@@ -264,7 +269,6 @@ int prepare_ethash(const hf_ethash_args &a, Prepared &p) {
   d.pow2_mask = (d.n_items & (d.n_items - 1)) == 0 ? d.n_items - 1 : 0;
   d.target = g_const.eth_target;
   std::memcpy(d.header, g_const.eth_header, sizeof d.header);
-  static_assert(sizeof(EthashDevArgs) <= sizeof(p.blob), "blob too small");
   std::memcpy(p.blob, &d, sizeof d);
   p.exact_grid = true;
   return HF_OK;
@@ -667,9 +671,13 @@ HF_API int hf_time_pair(const hf_plan *plan, int mode, const void *const *args1,
   auto once = [&](int i) -> int {
     const int s = i % nsets;
     int rc = HF_OK;
-    if (mode == 0 || mode == 2) rc = do_launch_native(plan->ids[0], p1[s], mode == 2 ? 0 : grid_blocks, b1, stream);
+    // A kernel whose grid fixes its amount of work (ethash) always gets grid_blocks; the
+    // others size their own grid in the back-to-back mode.
+    const int g1 = (mode == 2 && !p1[s].exact_grid) ? 0 : grid_blocks;
+    const int g2 = (mode == 2 && !p2[s].exact_grid) ? 0 : grid_blocks;
+    if (mode == 0 || mode == 2) rc = do_launch_native(plan->ids[0], p1[s], g1, b1, stream);
     if (rc != HF_OK) return rc;
-    if (mode == 1 || mode == 2) rc = do_launch_native(plan->ids[1], p2[s], mode == 2 ? 0 : grid_blocks, b2, stream);
+    if (mode == 1 || mode == 2) rc = do_launch_native(plan->ids[1], p2[s], g2, b2, stream);
     if (rc != HF_OK) return rc;
     if (mode == 3) rc = do_launch_fused(plan, p1[s], p2[s], grid_blocks, stream);
     return rc;
