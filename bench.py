@@ -52,15 +52,17 @@ def parse():
 class TensorPair:
     """One tensor pair: `nsets` independent input/output sets so repeats miss the last-level cache."""
 
-    def __init__(self, name, k1, k2, make_set, bytes1, bytes2, min_footprint=1 << 30):
+    def __init__(self, name, k1, k2, make_set, bytes1, bytes2, min_read_footprint=600 << 20):
+        # Enough sets that even the smaller of the two read streams cycles through more bytes
+        # than the 256 MB memory-side cache holds, so neither kernel re-reads cached inputs.
         self.name, self.k1, self.k2 = name, k1, k2
         self.bytes1, self.bytes2 = bytes1, bytes2
         self.sets = []
-        footprint = 0
-        while footprint < min_footprint or len(self.sets) < 2:
+        read_footprint = 0
+        while read_footprint < min_read_footprint or len(self.sets) < 2:
             s = make_set(len(self.sets))
             self.sets.append(s)
-            footprint += s["footprint"]
+            read_footprint += s["min_read"]
         self.args1 = [s["a1"] for s in self.sets]
         self.args2 = [s["a2"] for s in self.sets]
 
@@ -92,7 +94,7 @@ def build_tensor_pairs(names):
             y = rand((32, 64, 112, 112), SEED + 10 * i + 1)
             val = torch.empty((32, 64, 56, 56), device="cuda")
             idx = torch.empty((32, 64, 56, 56), dtype=torch.int64, device="cuda")
-            return dict(keep=(x, col, y, val, idx), footprint=nbytes(x, col, y, val, idx),
+            return dict(keep=(x, col, y, val, idx), min_read=min(nbytes(x), nbytes(y)),
                         a1=H.im2col_args(x, col), a2=H.maxpool_args(y, val, idx, (3, 3), (2, 2), (1, 1)))
         pairs["im2col_maxpool"] = TensorPair("im2col_maxpool", "im2col_kernel", "MaxPoolForward", mk,
                                              256901120, 179830784)
@@ -103,7 +105,7 @@ def build_tensor_pairs(names):
             inv = torch.empty(256, device="cuda")
             u = rand((32, 64, 56, 56), SEED + 10 * i + 3)
             out = torch.empty((32, 64, 112, 112), device="cuda")
-            return dict(keep=(x, mean, inv, u, out), footprint=nbytes(x, u, out),
+            return dict(keep=(x, mean, inv, u, out), min_read=min(nbytes(x), nbytes(u)),
                         a1=H.bn_stats_args(x, mean, inv, 1e-5, 0.0), a2=H.upsample_nearest_args(u, out))
         pairs["bn_upsample"] = TensorPair("bn_upsample", "batch_norm_collect_statistics_kernel",
                                           "upsample_nearest2d_out_frame", mk, 25692160, 128450560)
@@ -114,7 +116,7 @@ def build_tensor_pairs(names):
             y = rand((16, 128, 64, 64), SEED + 10 * i + 5)
             val = torch.empty((16, 128, 32, 32), device="cuda")
             idx = torch.empty((16, 128, 32, 32), dtype=torch.int64, device="cuda")
-            return dict(keep=(x, hist, y, val, idx), footprint=nbytes(x, y, val, idx),
+            return dict(keep=(x, hist, y, val, idx), min_read=min(nbytes(x), nbytes(y)),
                         a1=H.histc_args(x, hist, 1024, 0.0, 1.0), a2=H.maxpool_args(y, val, idx, (2, 2), (2, 2), (0, 0)))
         pairs["histc_maxpool"] = TensorPair("histc_maxpool", "kernelHistogram1D", "MaxPoolForward", mk,
                                             268439552, 58720256)

@@ -3,6 +3,7 @@
 #include <hip/hip_runtime.h>
 
 #include <algorithm>
+#include <cmath>
 #include <cstring>
 #include <fstream>
 #include <mutex>
@@ -191,7 +192,7 @@ int prepare_maxpool(const hf_maxpool_args &a, Prepared &p) {
     return fail(HF_EINVAL, "MaxPoolForward: last window starts outside the input");
   std::memcpy(p.blob, &a, sizeof a);
   const bool common = a.stride_h == 2 && a.stride_w == 2 && a.dilation_h == 1 && a.dilation_w == 1 &&
-                      a.width % 8 == 0 && a.pooled_width * 2 == a.width && a.pooled_width % 4 == 0 &&
+                      a.width % 4 == 0 && a.pooled_width * 2 == a.width && a.pooled_width % 2 == 0 &&
                       aligned16(a.bottom_data) && aligned16(a.top_data) && aligned16(a.top_mask) &&
                       (int64_t)a.num * a.channels * a.height * a.width < (int64_t)1 << 31;
   p.hint = HINT_GENERIC;
@@ -201,7 +202,7 @@ int prepare_maxpool(const hf_maxpool_args &a, Prepared &p) {
   if (common && a.kernel_h == 2 && a.kernel_w == 2 && a.pad_h == 0 && a.pad_w == 0 &&
       a.pooled_height == (a.height - 2) / 2 + 1)
     p.hint = HINT_POOL_K2S2P0;
-  p.items = p.hint ? (unsigned long long)a.nthreads / 4 : (unsigned long long)a.nthreads;
+  p.items = p.hint ? (unsigned long long)a.nthreads / 2 : (unsigned long long)a.nthreads;
   return HF_OK;
 }
 
@@ -231,10 +232,10 @@ int prepare_upsample(const hf_upsample_nearest_args &a, Prepared &p) {
     return fail(HF_EINVAL, "upsample_nearest2d_out_frame: scale must be positive");
   std::memcpy(p.blob, &a, sizeof a);
   const bool fast = a.height2 == 2 * a.height1 && a.width2 == 2 * a.width1 && a.height_scale == 0.5f &&
-                    a.width_scale == 0.5f && a.width1 % 4 == 0 && aligned16(a.idata) && aligned16(a.odata) &&
+                    a.width_scale == 0.5f && a.width1 % 2 == 0 && aligned16(a.idata) && aligned16(a.odata) &&
                     a.nc * a.height2 * a.width2 < (size_t)1 << 32;
   p.hint = fast ? HINT_UP_2X : HINT_GENERIC;
-  p.items = fast ? a.nc * a.height1 * (a.width1 / 4) : a.nc * a.height2 * a.width2;
+  p.items = fast ? a.nc * a.height1 * (a.width1 / 2) : a.nc * a.height2 * a.width2;
   return HF_OK;
 }
 
@@ -251,7 +252,11 @@ int prepare_histc(const hf_histc_args &a, Prepared &p) {
   if (a.nbins > 15360) return fail(HF_EUNSUPPORTED, "kernelHistogram1D: more bins than fit the LDS budget (15360)");
   std::memcpy(p.blob, &a, sizeof a);
   const bool fast = a.b.strides[0] == 1 && aligned16(a.b.data);
-  p.hint = fast ? HINT_HIST_VEC4 : HINT_GENERIC;
+  // max - min a power of two (exact reciprocal): the division in the bin formula can be a multiply
+  int exp2 = 0;
+  const float range = a.maxvalue - a.minvalue;
+  const bool pow2 = std::frexp(range, &exp2) == 0.5f && exp2 > -100 && exp2 < 100;
+  p.hint = (fast ? HINT_HIST_VEC4 : HINT_GENERIC) | (pow2 ? HINT_HIST_POW2 : 0);
   p.lds = (unsigned)a.nbins * 4u;
   p.items = fast ? (unsigned long long)(a.total_elements + 3) / 4 : (unsigned long long)a.total_elements;
   return HF_OK;
@@ -332,13 +337,17 @@ unsigned long long wanted_blocks(const Prepared &p, unsigned threads) {
   return (p.items + threads - 1) / threads;
 }
 
-// Default grid: enough resident workgroups to fill every CU twice over, never
-// more than the work asks for.  Streaming bodies stride over the rest.
-unsigned default_grid(unsigned long long want, unsigned block_threads) {
+// Default grid of one kernel inside a block of `block_threads` threads: enough workgroups
+// to fill every CU eight times over, never more than the work asks for.  The streaming
+// bodies stride over the rest; a larger grid evens out their tail.  The histogram is the
+// exception: every block flushes its LDS bins with one global atomic per bin, so it runs
+// one block per CU and keeps eight loads per lane in flight instead.
+unsigned default_grid(const Prepared &p, unsigned own_threads, unsigned block_threads) {
+  const unsigned long long want = wanted_blocks(p, own_threads);
   const unsigned per_cu = std::max(1u, 2048u / block_threads);
-  const unsigned long long cap = (unsigned long long)cu_count() * per_cu * 2ull;
-  unsigned long long g = std::min(std::max(want, 1ull), cap);
-  return (unsigned)g;
+  const unsigned long long cap =
+      p.id == K_HISTC ? (unsigned long long)cu_count() : (unsigned long long)cu_count() * per_cu * 8ull;
+  return (unsigned)std::min(std::max(want, 1ull), cap);
 }
 
 constexpr unsigned kDefaultEthashGrid = 8192;  // the authors' launches: scripts/data/ethminer_event.csv
@@ -349,7 +358,7 @@ int do_launch_native(KernelId id, const Prepared &p, int grid_blocks, unsigned b
   unsigned grid;
   if (grid_blocks > 0) grid = (unsigned)grid_blocks;
   else if (p.exact_grid) grid = kDefaultEthashGrid;
-  else grid = default_grid(wanted_blocks(p, block), block);
+  else grid = default_grid(p, block, block);
   if (!p.exact_grid && p.items == 0) return HF_OK;  // nothing to do
   hipError_t e = is_crypto(id) ? launch_native_crypto(id, p.blob, p.hint, grid, block, p.lds, stream)
                                : launch_native_dl(id, p.blob, p.hint, grid, block, p.lds, stream);
@@ -370,6 +379,7 @@ struct hf_plan {
   const Preset *preset;
   Partition part;
   int barrier_mode;
+  unsigned grid_override[2] = {0, 0};  // hf_plan_set_grids
 };
 
 // ------------------------------------------------------------------ C-ABI
@@ -513,6 +523,14 @@ HF_API int hf_plan_set_barrier_mode(hf_plan *plan, int mode) {
   return HF_OK;
 }
 
+HF_API int hf_plan_set_grids(hf_plan *plan, int grid1, int grid2) {
+  if (!plan) return fail(HF_EINVAL, "null plan");
+  if (grid1 < 0 || grid2 < 0) return fail(HF_EINVAL, "negative grid");
+  plan->grid_override[0] = (unsigned)grid1;
+  plan->grid_override[1] = (unsigned)grid2;
+  return HF_OK;
+}
+
 HF_API void hf_plan_free(hf_plan *plan) { delete plan; }
 
 HF_API int hf_plan_partition(const hf_plan *plan, hf_partition *out) {
@@ -613,14 +631,13 @@ int do_launch_fused(const hf_plan *plan, const Prepared &p1, const Prepared &p2,
   g.hint2 = p2.hint;
   g.grid1 = g.grid2 = 0;
   const bool crypto = is_crypto(plan->ids[0]);
-  const unsigned long long w1 = p1.exact_grid ? 0 : wanted_blocks(p1, g.d1);
-  const unsigned long long w2 = p2.exact_grid ? 0 : wanted_blocks(p2, g.d2);
+  const unsigned exact = grid_blocks > 0 ? (unsigned)grid_blocks : kDefaultEthashGrid;
   hipError_t e;
   if (plan->barrier_mode == HF_BARRIER_BLOCKIDX) {
     // Each kernel gets its own workgroups inside one launch.
     const unsigned block = std::max(g.d1, g.d2);
-    g.grid1 = p1.exact_grid ? (grid_blocks > 0 ? (unsigned)grid_blocks : kDefaultEthashGrid) : default_grid(w1, block);
-    g.grid2 = p2.exact_grid ? (grid_blocks > 0 ? (unsigned)grid_blocks : kDefaultEthashGrid) : default_grid(w2, block);
+    g.grid1 = p1.exact_grid ? exact : default_grid(p1, g.d1, block);
+    g.grid2 = p2.exact_grid ? exact : default_grid(p2, g.d2, block);
     if (!p1.exact_grid && !p2.exact_grid && grid_blocks > 0) {
       g.grid1 = std::max(1u, (unsigned)grid_blocks / 2);
       g.grid2 = std::max(1u, (unsigned)grid_blocks - g.grid1);
@@ -629,10 +646,19 @@ int do_launch_fused(const hf_plan *plan, const Prepared &p1, const Prepared &p2,
     e = crypto ? launch_fused_crypto(plan->ids[0], plan->ids[1], MODE_BLOCKIDX, p1.blob, p2.blob, g, g.grid1 + g.grid2, lds, stream)
                : launch_fused_dl(plan->ids[0], plan->ids[1], MODE_BLOCKIDX, p1.blob, p2.blob, g, g.grid1 + g.grid2, lds, stream);
   } else {
-    unsigned grid;
-    if (grid_blocks > 0) grid = (unsigned)grid_blocks;
-    else if (p1.exact_grid || p2.exact_grid) grid = kDefaultEthashGrid;
-    else grid = default_grid(std::max(w1, w2), g.d1 + g.d2);
+    // One grid for both halves.  When the caller names it, both halves stride over all of it
+    // (a kernel whose grid fixes its work, ethash, always does); otherwise each half strides
+    // over its own preferred number of blocks and the launch covers the larger of the two.
+    const unsigned block = g.d1 + g.d2;
+    if (grid_blocks > 0) {
+      g.grid1 = g.grid2 = (unsigned)grid_blocks;
+    } else {
+      g.grid1 = p1.exact_grid ? exact : default_grid(p1, g.d1, block);
+      g.grid2 = p2.exact_grid ? exact : default_grid(p2, g.d2, block);
+      if (plan->grid_override[0] && !p1.exact_grid) g.grid1 = plan->grid_override[0];
+      if (plan->grid_override[1] && !p2.exact_grid) g.grid2 = plan->grid_override[1];
+    }
+    const unsigned grid = std::max(g.grid1, g.grid2);
     const size_t lds = 4 * kBarrierWords + g.lds1 + g.lds2;
     const FuseMode mode = plan->barrier_mode == HF_BARRIER_MATCHED ? MODE_MATCHED : MODE_HFUSE;
     e = crypto ? launch_fused_crypto(plan->ids[0], plan->ids[1], mode, p1.blob, p2.blob, g, grid, lds, stream)

@@ -13,10 +13,19 @@
 namespace hfuse {
 
 // Hints (0 always means the general path).
-enum { HINT_GENERIC = 0, HINT_IM2COL_3X3_S1P1 = 1, HINT_POOL_K3S2P1 = 1, HINT_POOL_K2S2P0 = 2, HINT_UP_2X = 1, HINT_BN_VEC4 = 1, HINT_HIST_VEC4 = 1 };
+enum { HINT_GENERIC = 0, HINT_IM2COL_3X3_S1P1 = 1, HINT_POOL_K3S2P1 = 1, HINT_POOL_K2S2P0 = 2, HINT_UP_2X = 1, HINT_BN_VEC4 = 1, HINT_HIST_VEC4 = 1, HINT_HIST_POW2 = 2 };
 
 __device__ __forceinline__ f32x4 ld4(const float *p) { return *reinterpret_cast<const f32x4 *>(p); }
-__device__ __forceinline__ void st4(float *p, f32x4 v) { __builtin_nontemporal_store(v, reinterpret_cast<f32x4 *>(p)); }
+#ifndef HF_NT_STORES
+#define HF_NT_STORES 1
+#endif
+__device__ __forceinline__ void st4(float *p, f32x4 v) {
+#if HF_NT_STORES
+  __builtin_nontemporal_store(v, reinterpret_cast<f32x4 *>(p));
+#else
+  *reinterpret_cast<f32x4 *>(p) = v;
+#endif
+}
 
 // ----------------------------------------------------------------------------
 // im2col_kernel<float>  (argument list: scripts/data/ml-event.csv:17)
@@ -113,8 +122,8 @@ struct MaxPoolBody {
 
   template <class SB>
   static __device__ void run(const Args &a, SB &sb, unsigned char *, unsigned hint) {
-    if (hint == HINT_POOL_K3S2P1) { vec4_s2<3, 1>(a, sb); return; }
-    if (hint == HINT_POOL_K2S2P0) { vec4_s2<2, 0>(a, sb); return; }
+    if (hint == HINT_POOL_K3S2P1) { vec2_s2<3, 1>(a, sb); return; }
+    if (hint == HINT_POOL_K2S2P0) { vec2_s2<2, 0>(a, sb); return; }
     const int64_t stride = (int64_t)sb.nblocks * sb.nthreads;
     for (int64_t index = (int64_t)sb.bid * sb.nthreads + sb.tid; index < a.nthreads; index += stride) {
       const int pw = (int)(index % a.pooled_width);
@@ -143,70 +152,83 @@ struct MaxPoolBody {
     }
   }
 
-  // K x K window, stride 2, pad P (K=3,P=1 or K=2,P=0), width % 8 == 0 and
-  // pooled_width == width/2: a work item owns four neighbouring outputs and
-  // reads, per window row, two aligned 16-byte vectors (+ the left edge for P=1).
+  // K x K window, stride 2, pad P (K=3,P=1 or K=2,P=0), width % 4 == 0 and
+  // pooled_width == width/2: a work item owns two neighbouring outputs and reads,
+  // per window row, one aligned 16-byte vector (+ the left edge for P=1).  Two
+  // outputs per lane make every store instruction of the wave one contiguous
+  // run (8 B of values, 16 B of int64 indices per lane): write-once streams
+  // leave the chip as whole lines.
   template <int K, int P, class SB>
-  static __device__ __forceinline__ void vec4_s2(const Args &a, SB &sb) {
+  static __device__ __forceinline__ void vec2_s2(const Args &a, SB &sb) {
     const unsigned W = (unsigned)a.width, H = (unsigned)a.height;
     const unsigned PW = (unsigned)a.pooled_width, PH = (unsigned)a.pooled_height;
-    const unsigned pq = PW >> 2;
-    const unsigned n4 = (unsigned)a.nthreads >> 2;
+    const unsigned ph2 = PW >> 1;
+    const unsigned n2 = (unsigned)a.nthreads >> 1;
     const unsigned stride = sb.nblocks * sb.nthreads;
-    for (unsigned idx4 = sb.bid * sb.nthreads + sb.tid; idx4 < n4; idx4 += stride) {
-      const unsigned pw4 = idx4 % pq;
-      const unsigned t = idx4 / pq;
+    for (unsigned idx2 = sb.bid * sb.nthreads + sb.tid; idx2 < n2; idx2 += stride) {
+      const unsigned pw2 = idx2 % ph2;
+      const unsigned t = idx2 / ph2;
       const unsigned ph = t % PH;
       const unsigned nc = t / PH;
       const float *plane = a.bottom_data + (size_t)nc * H * W;
       const int hstart = (int)ph * 2 - P;
-      const unsigned wbase = pw4 << 3;
-      float maxv[4];
-      int maxi[4];
+      const unsigned wbase = pw2 << 2;
+      float maxv[2];
+      int maxi[2];
       const int h0 = hstart < 0 ? 0 : hstart;
 #pragma unroll
-      for (int o = 0; o < 4; o++) {
+      for (int o = 0; o < 2; o++) {
         const int ws = (int)wbase + 2 * o - P;
         maxv[o] = -INFINITY;
         maxi[o] = h0 * (int)W + (ws < 0 ? 0 : ws);
+      }
+      // issue every row's loads before the compare chain
+      f32x4 v[K];
+      float left[K];
+#pragma unroll
+      for (int i = 0; i < K; i++) {
+        const int h = hstart + i;
+        const bool in = h >= 0 && h < (int)H;
+        const float *row = plane + (unsigned)(in ? h : h0) * W + wbase;
+        v[i] = ld4(row);
+        left[i] = (P == 1 && wbase > 0) ? row[-1] : 0.0f;
       }
 #pragma unroll
       for (int i = 0; i < K; i++) {
         const int h = hstart + i;
         if (h < 0 || h >= (int)H) continue;
-        const float *row = plane + (unsigned)h * W + wbase;
-        const f32x4 v0 = ld4(row), v1 = ld4(row + 4);
-        float vals[9];
         // vals[k] is input column wbase - P + k
+        float vals[5];
         if (P == 1) {
-          vals[0] = wbase > 0 ? row[-1] : 0.0f;
-          vals[1] = v0.x; vals[2] = v0.y; vals[3] = v0.z; vals[4] = v0.w;
-          vals[5] = v1.x; vals[6] = v1.y; vals[7] = v1.z; vals[8] = v1.w;
+          vals[0] = left[i]; vals[1] = v[i].x; vals[2] = v[i].y; vals[3] = v[i].z; vals[4] = v[i].w;
         } else {
-          vals[0] = v0.x; vals[1] = v0.y; vals[2] = v0.z; vals[3] = v0.w;
-          vals[4] = v1.x; vals[5] = v1.y; vals[6] = v1.z; vals[7] = v1.w;
-          vals[8] = 0.0f;
+          vals[0] = v[i].x; vals[1] = v[i].y; vals[2] = v[i].z; vals[3] = v[i].w; vals[4] = 0.0f;
         }
         const int base_idx = h * (int)W + (int)wbase - P;
 #pragma unroll
-        for (int o = 0; o < 4; o++)
+        for (int o = 0; o < 2; o++)
 #pragma unroll
           for (int j = 0; j < K; j++) {
             const int k = 2 * o + j;
             if (P == 1 && k == 0 && wbase == 0) continue;  // column -1 is padding
-            const float v = vals[k];
-            if ((v > maxv[o]) || isnan(v)) {
-              maxv[o] = v;
+            const float x = vals[k];
+            if ((x > maxv[o]) || isnan(x)) {
+              maxv[o] = x;
               maxi[o] = base_idx + k;
             }
           }
       }
-      f32x4 ov = {maxv[0], maxv[1], maxv[2], maxv[3]};
-      st4(a.top_data + (size_t)idx4 * 4, ov);
-      i64x2 *mp = reinterpret_cast<i64x2 *>(a.top_mask + (size_t)idx4 * 4);
-      i64x2 m0 = {maxi[0], maxi[1]}, m1 = {maxi[2], maxi[3]};
-      __builtin_nontemporal_store(m0, mp);
-      __builtin_nontemporal_store(m1, mp + 1);
+      const f32x2 ov = {maxv[0], maxv[1]};
+      const i64x2 om = {maxi[0], maxi[1]};
+      f32x2 *vp = reinterpret_cast<f32x2 *>(a.top_data + (size_t)idx2 * 2);
+      i64x2 *mp = reinterpret_cast<i64x2 *>(a.top_mask + (size_t)idx2 * 2);
+#if HF_NT_STORES
+      __builtin_nontemporal_store(ov, vp);
+      __builtin_nontemporal_store(om, mp);
+#else
+      *vp = ov;
+      *mp = om;
+#endif
     }
   }
 };
@@ -221,22 +243,34 @@ struct UpsampleNearestBody {
   template <class SB>
   static __device__ void run(const Args &a, SB &sb, unsigned char *, unsigned hint) {
     if (hint == HINT_UP_2X) {
-      // Exact 2x: one 16-byte load feeds two output rows of two 16-byte stores each.
-      const unsigned w1q = (unsigned)a.width1 >> 2;
-      const unsigned h1 = (unsigned)a.height1;
+      // Exact 2x: a lane loads two neighbouring input pixels (8 B) and stores the four
+      // output pixels they expand to (16 B) into both output rows, so each load and each
+      // store instruction of the wave covers one contiguous run.  Two items per trip keep
+      // two loads in flight.
+      const unsigned w1h = (unsigned)a.width1 >> 1;
       const unsigned w2 = (unsigned)a.width2;
-      const unsigned n4 = (unsigned)(a.nc * a.height1) * w1q;
+      const unsigned n2 = (unsigned)(a.nc * a.height1) * w1h;
       const unsigned stride = sb.nblocks * sb.nthreads;
-      for (unsigned idx = sb.bid * sb.nthreads + sb.tid; idx < n4; idx += stride) {
-        const unsigned x4 = idx % w1q;
-        const unsigned row = idx / w1q;  // c * h1 + y1
-        const f32x4 v = ld4(a.idata + (size_t)idx * 4);
-        // output row index: c*h2 + 2*y1 = 2*(c*h1 + y1)
-        float *o = a.odata + (size_t)row * 2u * w2 + (size_t)x4 * 8u;
-        const f32x4 lo = {v.x, v.x, v.y, v.y}, hi = {v.z, v.z, v.w, v.w};
-        st4(o, lo); st4(o + 4, hi);
-        st4(o + w2, lo); st4(o + w2 + 4, hi);
-        (void)h1;
+      const f32x2 *in = reinterpret_cast<const f32x2 *>(a.idata);
+      for (unsigned idx = sb.bid * sb.nthreads + sb.tid; idx < n2; idx += 2 * stride) {
+        const unsigned idx_b = idx + stride;
+        const bool has_b = idx_b < n2;
+        const f32x2 va = in[idx];
+        const f32x2 vb = has_b ? in[idx_b] : f32x2{0.0f, 0.0f};
+        {
+          const unsigned xh = idx % w1h, row = idx / w1h;  // row = c * h1 + y1; output row = 2 * row
+          float *o = a.odata + (size_t)row * 2u * w2 + (size_t)xh * 4u;
+          const f32x4 e = {va.x, va.x, va.y, va.y};
+          st4(o, e);
+          st4(o + w2, e);
+        }
+        if (has_b) {
+          const unsigned xh = idx_b % w1h, row = idx_b / w1h;
+          float *o = a.odata + (size_t)row * 2u * w2 + (size_t)xh * 4u;
+          const f32x4 e = {vb.x, vb.x, vb.y, vb.y};
+          st4(o, e);
+          st4(o + w2, e);
+        }
       }
       return;
     }
@@ -314,19 +348,30 @@ struct BnStatsBody {
         const unsigned chunks = (unsigned)N * lq;
         const float *base = a.input.data + (size_t)plane * a.input.strides[1];
         float k = 0.0f;
-        for (unsigned ch = sb.tid; ch < chunks; ch += sb.nthreads) {
-          const unsigned b = ch / lq, q = ch - b * lq;
-          const f32x4 v = ld4(base + (size_t)b * a.input.strides[0] + (size_t)q * 4);
-          // Welford of the chunk, then merge (4, m4, s4) into the running triple.
+        // Welford of a chunk of four, then merge (4, m4, s4) into the running triple.
+        auto merge4 = [&](const f32x4 v) {
           const float m4 = (v.x + v.y + v.z + v.w) * 0.25f;
           const float dx = v.x - m4, dy = v.y - m4, dz = v.z - m4, dw = v.w - m4;
           const float s4 = dx * dx + dy * dy + dz * dz + dw * dw;
           k += 1.0f;
-          const float inv = __frcp_rn(k);           // 4 / (4k)
+          const float inv = __frcp_rn(k);  // 4 / (4k)
           const float d = m4 - acc.mean;
           acc.mean += d * inv;
           acc.m2 += s4 + d * d * (4.0f * (k - 1.0f)) * inv;
+        };
+        auto chunk = [&](unsigned ch) {
+          const unsigned b = ch / lq, q = ch - b * lq;
+          return ld4(base + (size_t)b * a.input.strides[0] + (size_t)q * 4);
+        };
+        unsigned ch = sb.tid;
+        for (; ch + 3 * sb.nthreads < chunks; ch += 4 * sb.nthreads) {  // four loads in flight
+          f32x4 v[4];
+#pragma unroll
+          for (int u = 0; u < 4; u++) v[u] = chunk(ch + u * sb.nthreads);
+#pragma unroll
+          for (int u = 0; u < 4; u++) merge4(v[u]);
         }
+        for (; ch < chunks; ch += sb.nthreads) merge4(chunk(ch));
         acc.n = 4.0f * k;
       } else {
         const int total = N * L;
@@ -366,9 +411,15 @@ struct HistcBody {
   using Args = hf_histc_args;
   static constexpr bool kBarriers = true;
 
-  static __device__ __forceinline__ void count(unsigned *bins, float v, float lo, float hi, float scale_n, float range, int nbins) {
+  // bin = (int)((v - min) * nbins / (max - min)) in fp32, bin == nbins -> nbins - 1.
+  // POW2: max - min is a power of two, so the correctly rounded division equals the
+  // multiplication by its (exact) reciprocal and the IEEE division sequence is not needed.
+  template <bool POW2>
+  static __device__ __forceinline__ void count(unsigned *bins, float v, float lo, float hi, float scale_n, float range,
+                                               float inv_range, int nbins) {
     if (v >= lo && v <= hi) {
-      int bin = (int)((v - lo) * scale_n / range);
+      const float t = (v - lo) * scale_n;
+      int bin = (int)(POW2 ? t * inv_range : t / range);
       if (bin == nbins) bin -= 1;
       __hip_atomic_fetch_add(bins + bin, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
     }
@@ -376,30 +427,50 @@ struct HistcBody {
 
   template <class SB>
   static __device__ void run(const Args &a, SB &sb, unsigned char *lds, unsigned hint) {
+    if (hint & HINT_HIST_POW2) body<true>(a, sb, lds, hint);
+    else body<false>(a, sb, lds, hint);
+  }
+
+  template <bool POW2, class SB>
+  static __device__ __forceinline__ void body(const Args &a, SB &sb, unsigned char *lds, unsigned hint) {
     unsigned *bins = reinterpret_cast<unsigned *>(lds);
     const int nbins = a.nbins;
     for (int i = (int)sb.tid; i < nbins; i += (int)sb.nthreads) bins[i] = 0;
     sb.sync();
     const float lo = a.minvalue, hi = a.maxvalue, range = hi - lo, fn = (float)nbins;
+    const float inv_range = 1.0f / range;
     const float *b = a.b.data;
     const int64_t total = a.total_elements;
-    if (hint == HINT_HIST_VEC4) {
+    auto count4 = [&](const f32x4 v) {
+      count<POW2>(bins, v.x, lo, hi, fn, range, inv_range, nbins);
+      count<POW2>(bins, v.y, lo, hi, fn, range, inv_range, nbins);
+      count<POW2>(bins, v.z, lo, hi, fn, range, inv_range, nbins);
+      count<POW2>(bins, v.w, lo, hi, fn, range, inv_range, nbins);
+    };
+    if (hint & HINT_HIST_VEC4) {
       const int64_t n4 = total >> 2;
       const int64_t stride = (int64_t)sb.nblocks * sb.nthreads;
-      for (int64_t i = (int64_t)sb.bid * sb.nthreads + sb.tid; i < n4; i += stride) {
-        const f32x4 v = ld4(b + i * 4);
-        count(bins, v.x, lo, hi, fn, range, nbins);
-        count(bins, v.y, lo, hi, fn, range, nbins);
-        count(bins, v.z, lo, hi, fn, range, nbins);
-        count(bins, v.w, lo, hi, fn, range, nbins);
+      int64_t i = (int64_t)sb.bid * sb.nthreads + sb.tid;
+      // several 16-byte loads in flight per lane before the dependent LDS atomics
+#ifndef HF_HIST_U
+#define HF_HIST_U 8
+#endif
+      for (; i + (HF_HIST_U - 1) * stride < n4; i += HF_HIST_U * stride) {
+        f32x4 v[HF_HIST_U];
+#pragma unroll
+        for (int u = 0; u < HF_HIST_U; u++) v[u] = ld4(b + (i + u * stride) * 4);
+#pragma unroll
+        for (int u = 0; u < HF_HIST_U; u++) count4(v[u]);
       }
+      for (; i < n4; i += stride) count4(ld4(b + i * 4));
       if (sb.bid == 0)
-        for (int64_t i = (n4 << 2) + sb.tid; i < total; i += sb.nthreads) count(bins, b[i], lo, hi, fn, range, nbins);
+        for (int64_t k = (n4 << 2) + sb.tid; k < total; k += sb.nthreads)
+          count<POW2>(bins, b[k], lo, hi, fn, range, inv_range, nbins);
     } else {
       const int64_t stride = (int64_t)sb.nblocks * sb.nthreads;
       const int64_t bs = a.b.strides[0];
       for (int64_t i = (int64_t)sb.bid * sb.nthreads + sb.tid; i < total; i += stride)
-        count(bins, b[i * bs], lo, hi, fn, range, nbins);
+        count<POW2>(bins, b[i * bs], lo, hi, fn, range, inv_range, nbins);
     }
     sb.sync();
     const int64_t as = a.a.strides[0];

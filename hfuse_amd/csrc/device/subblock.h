@@ -65,7 +65,8 @@ struct FuseGeom {
   unsigned d1, d2;          // threads of each half
   unsigned lds1, lds2;      // LDS bytes of each half
   unsigned hint1, hint2;    // fast-path selector the host derived from each argument list
-  unsigned grid1, grid2;    // blockIdx mode: workgroups given to each kernel
+  unsigned grid1, grid2;    // workgroups each kernel strides over: in the fused kernel half k works in
+                            // blocks [0, grid_k) only; in blockIdx mode kernel 2 starts at block grid1
 };
 
 constexpr unsigned kBarrierWords = 4;  // 16 bytes reserved at the base of LDS for arrival counters
@@ -96,11 +97,16 @@ __global__ __launch_bounds__(T) void fused_kernel(typename K1::Args a1, typename
   const unsigned wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   constexpr int B1 = (kSubset && K1::kBarriers) ? BAR_SUBSET : BAR_WORKGROUP;
   constexpr int B2 = (kSubset && K2::kBarriers) ? BAR_SUBSET : BAR_WORKGROUP;
+  // Both halves see the launch's blockIdx (the reference leaves blockIdx/gridDim alone,
+  // include/ThreadInfoRewriter.h:29-31); a half whose kernel wants fewer workgroups than the
+  // launch has simply ends in the surplus blocks, which frees its wave slots for the partner.
   if (wave < (g.d1 >> 6)) {
-    SubBlock<B1> sb{tid, g.d1, blockIdx.x, gridDim.x, bars + 0, 0};
+    if (blockIdx.x >= g.grid1) return;
+    SubBlock<B1> sb{tid, g.d1, blockIdx.x, g.grid1, bars + 0, 0};
     K1::run(a1, sb, smem + 4 * kBarrierWords, g.hint1);
   } else {
-    SubBlock<B2> sb{tid - g.d1, g.d2, blockIdx.x, gridDim.x, bars + 1, 0};
+    if (blockIdx.x >= g.grid2) return;
+    SubBlock<B2> sb{tid - g.d1, g.d2, blockIdx.x, g.grid2, bars + 1, 0};
     K2::run(a2, sb, smem + 4 * kBarrierWords + g.lds1, g.hint2);
   }
 }

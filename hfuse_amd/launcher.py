@@ -40,8 +40,8 @@ class Config:
         return self
 
     def __del__(self):
-        if getattr(self, "_h", None):
-            L.lib().hf_config_free(self._h)
+        if getattr(self, "_h", None) and L is not None and L._lib is not None:
+            L._lib.hf_config_free(self._h)
             self._h = None
 
     @property
@@ -89,8 +89,8 @@ class Plan:
                                      C.byref(self._h)))
 
     def __del__(self):
-        if getattr(self, "_h", None):
-            L.lib().hf_plan_free(self._h)
+        if getattr(self, "_h", None) and L is not None and L._lib is not None:
+            L._lib.hf_plan_free(self._h)
             self._h = None
 
     @property
@@ -105,6 +105,9 @@ class Plan:
 
     def set_barrier_mode(self, mode: int) -> None:
         check(L.lib().hf_plan_set_barrier_mode(self._h, mode))
+
+    def set_grids(self, grid1: int = 0, grid2: int = 0) -> None:
+        check(L.lib().hf_plan_set_grids(self._h, grid1, grid2))
 
     def local_index(self, half: int, tid: int):
         out = L.Dim3()

@@ -138,6 +138,14 @@ HF_API void hf_plan_free(hf_plan *plan);
  * then share the hardware barrier); HF_BARRIER_BLOCKIDX is always legal.
  */
 HF_API int hf_plan_set_barrier_mode(hf_plan *plan, int mode);
+/*
+ * Per-half grids of the fused launch when the caller leaves grid_blocks <= 0:
+ * half k strides over blocks [0, grid_k) and the launch covers max(grid1, grid2)
+ * blocks.  0 keeps the library's choice for that half.  (The reference's halves
+ * share the launch grid; a half that wants fewer blocks simply ends early in
+ * the surplus ones.)
+ */
+HF_API int hf_plan_set_grids(hf_plan *plan, int grid1, int grid2);
 HF_API int hf_plan_partition(const hf_plan *plan, hf_partition *out);
 /* Number of variants the reference's split loop would print (main.cpp:221-223). */
 HF_API int hf_plan_num_splits(const hf_config *cfg, int fusion_index);
