@@ -25,7 +25,10 @@ ROOT = os.path.dirname(os.path.abspath(__file__))
 sys.path.insert(0, ROOT)
 
 HBM_PEAK_GBPS = 8000.0            # MI355X HBM3E
-VALU_PEAK_GOPS = 256 * 64 * 2.4   # 256 CUs x 64 lanes x 2.4 GHz int32 op/s, in Gop/s
+VALU_PEAK_GOPS = 256 * 128 * 2.4  # 256 CUs x 128 lanes x 2.4 GHz int32 op/s in Gop/s (= 157.3 TFLOP/s fp32 / 2)
+# HBM bytes per launch of the headline fused kernel from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE, each
+# scaled by what the same counter reads for the plain copy kernel (profiles/bn_upsample_fused_hbm_traffic.md)
+HEADLINE_TRAFFIC_BYTES = {"bn_upsample": 157.22e6}
 SEED = 0x48467573
 
 # textbook primitive-op counts per hash (add / logic / rotate / shift = 1 each)
@@ -42,9 +45,13 @@ def parse():
     ap.add_argument("--pairs", default="all", help="comma list of pair names, or 'all'")
     ap.add_argument("--headline", default="bn_upsample")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
-    ap.add_argument("--no-sweep", action="store_true", help="time the table split only")
+    ap.add_argument("--sweep", action="store_true",
+                    help="also time every split of the reference's enumeration and report the fastest "
+                         "(default: the tuned split of the shipped fusion list)")
     ap.add_argument("--fused-only", action="store_true", help="launch only the fused kernel (profiling runs)")
     ap.add_argument("--search-log2", type=int, default=None, help="override log2 of the nonce ranges (debug)")
+    ap.add_argument("--calibrate-copy", type=int, default=0, metavar="MIB",
+                    help="also run the plain copy kernel on MIB mebibytes (the unit HBM counters are scaled by)")
     return ap.parse_args()
 
 
@@ -329,11 +336,20 @@ def main():
     hfuse_amd._lib.lib()  # fail loudly if the HIP library is missing
     torch.cuda.set_device(0)
     cfg = hfuse_amd.default_config()
+    if args.calibrate_copy:
+        from hfuse_amd import launcher as H
+        n = args.calibrate_copy * (1 << 20) // 4
+        src = [torch.rand(n, device="cuda") for _ in range(4)]
+        dst = [torch.empty(n, device="cuda") for _ in range(4)]
+        for i in range(12):
+            H.copy_f32(src[i % 4], dst[i % 4])
+        torch.cuda.synchronize()
+        del src, dst
     all_names = ["im2col_maxpool", "bn_upsample", "histc_maxpool", "sha256d_blake2b", "ethash_blake2b"]
     names = all_names if args.pairs == "all" else [n for n in args.pairs.split(",") if n]
     if args.headline not in names:
         names.append(args.headline)
-    sweep = not args.no_sweep
+    sweep = args.sweep
     report = {}
 
     # tensor pairs one at a time (each holds ~1 GiB of rotating buffers)
@@ -429,7 +445,7 @@ def main():
         "roofline": {"bound": "hbm", "achieved": (h["total_bytes"] / (h["event_ms_per_step"] * 1e-3) / 1e9) if h else None,
                      "peak": HBM_PEAK_GBPS, "unit": "GB/s",
                      "frac": (h["total_bytes"] / (h["event_ms_per_step"] * 1e-3) / 1e9 / HBM_PEAK_GBPS) if h else None,
-                     "traffic": None,
+                     "traffic": HEADLINE_TRAFFIC_BYTES.get(args.headline),
                      "kernel": h.get("fused_name"), "algorithmic_bytes_per_launch": h.get("total_bytes"),
                      "avg_launch_ms": h.get("event_ms_per_step")},
         "cpu_baseline": cpu,

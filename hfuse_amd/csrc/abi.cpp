@@ -345,8 +345,10 @@ unsigned long long wanted_blocks(const Prepared &p, unsigned threads) {
 unsigned default_grid(const Prepared &p, unsigned own_threads, unsigned block_threads) {
   const unsigned long long want = wanted_blocks(p, own_threads);
   const unsigned per_cu = std::max(1u, 2048u / block_threads);
-  const unsigned long long cap =
-      p.id == K_HISTC ? (unsigned long long)cu_count() : (unsigned long long)cu_count() * per_cu * 8ull;
+  // (two per CU when it shares its blocks with a partner that ends early)
+  const unsigned long long cap = p.id == K_HISTC
+                                     ? (unsigned long long)cu_count() * (own_threads == block_threads ? 1u : 2u)
+                                     : (unsigned long long)cu_count() * per_cu * 8ull;
   return (unsigned)std::min(std::max(want, 1ull), cap);
 }
 
@@ -482,6 +484,8 @@ HF_API int hf_plan_create(const hf_config *cfg, int fusion_index, const char *pr
     return fail(HF_EUNSUPPORTED, "pairs mixing a tensor kernel with a search kernel are not built");
   }
   std::string err;
+  if (split_idx == HF_SPLIT_TABLE && split_threads <= 0 && f.split > 0 && !p->base_line)
+    split_threads = (int)f.split;  // the pair's tuned default from the fusion list
   int rc = make_partition(plan->rows[0], plan->rows[1], *p, split_idx, split_threads, plan->part, err);
   if (rc != HF_OK) {
     delete plan;

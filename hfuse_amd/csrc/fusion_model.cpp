@@ -140,6 +140,18 @@ bool parse_config(const char *fusion_yaml, const char *kernels_yaml, Config &cfg
       if (!file || file->kind != YamlNode::Scalar) { err = "fusion list: " + at(n) + "missing required key 'File'"; return false; }
       if (!ks || ks->kind != YamlNode::Seq) { err = "fusion list: " + at(n) + "missing required key 'Kernels'"; return false; }
       f.file = file->scalar;
+      if (const YamlNode *sp = n.get("Split")) {
+        // not in the reference's schema: a tuned default for the thread partition of this pair
+        if (!to_uint(sp, f.split) || f.split == 0 || f.split % kWave != 0) {
+          err = "fusion list: " + at(*sp) + "'Split' must be a positive multiple of 64 threads";
+          return false;
+        }
+      }
+      for (auto &kv : n.map)
+        if (kv.first != "File" && kv.first != "Kernels" && kv.first != "Split") {
+          err = "fusion list: " + at(kv.second) + "unknown key '" + kv.first + "'";
+          return false;
+        }
       for (auto &k : ks->seq) {
         if (k.kind != YamlNode::Scalar) { err = "fusion list: " + at(k) + "kernel name must be a scalar"; return false; }
         f.kernels.push_back(k.scalar);

@@ -28,6 +28,7 @@ struct KernelRow {
 struct FusionRow {
   std::string file;
   std::vector<std::string> kernels;
+  uint32_t split = 0;  // optional `Split:` key: threads of kernel 1 when the caller asks for the table split
 };
 
 struct Config {

@@ -75,6 +75,9 @@ typedef struct {
  * and a string-keyed map of kernel rows.  `kernels_yaml` may also be the older
  * per-pair form, a bare sequence of rows (configs/im2col_maxpool.yaml); then
  * `fusion_yaml` may be NULL and the single fusion is that list in order.
+ * One key beyond the reference's schema is accepted in a fusion entry:
+ * `Split: <threads>`, a tuned default for kernel 1's share of the block, used
+ * when a plan is created with HF_SPLIT_TABLE.
  */
 HF_API int hf_config_load_text(const char *fusion_yaml, const char *kernels_yaml, hf_config **out);
 HF_API int hf_config_load_files(const char *fusion_path, const char *kernels_path, hf_config **out);

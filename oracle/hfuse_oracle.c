@@ -34,9 +34,15 @@
  *   Ethash hashimoto  : the light-client evaluation (cache + dataset items)
  *                       of libethash's published block-22 vector
  *                       (epoch 0, header 372eca24..., nonce 0x495732e0ed7a801c).
- *                       The search kernel's own record layout and its
- *                       "<= target" convention are this build's, not upstream's
- *                       (parity with ethminer@ae's Search_results unpinned).
+ *
+ * PARITY UNPINNED (only the un-vendored upstream sources could pin these):
+ *   - the record layout and hit policy of the three search kernels (ethminer@ae's
+ *     Search_results struct, ccminer's resNonces[0]/[1] slots and the digest word
+ *     each compares to its target): orc_hit and the "<= target" conventions of
+ *     orc_*_search are this build's own;
+ *   - PyTorch 1.4's histogram bin rounding for a general (min, max, nbins); for
+ *     power-of-two ranges such as (0, 1, 1024) the formula is exact and is
+ *     pinned against torch.histc.
  */
 #include <math.h>
 #include <stdint.h>
