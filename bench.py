@@ -327,7 +327,7 @@ def cpu_baseline_search(name, seconds=6.0):
 def main():
     args = parse()
     if args.gpus != 1:
-        print("bench.py: this build runs on one GPU (every pair shards without exchange; see DESIGN.md); "
+        print("bench.py: this build runs on one GPU only (every pair would shard without an exchange step); "
               "--gpus must be 1", file=sys.stderr)
         sys.exit(2)
     import torch
