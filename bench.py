@@ -142,23 +142,32 @@ def candidate_plans(cfg, k1, k2, sweep):
     return out
 
 
-def time_tensor_pair(cfg, pair, steps, warmup, sweep, fused_only):
-    """-> dict with per-launch milliseconds of native A, native B, back-to-back and the best fused split."""
+def time_tensor_pair(cfg, pair, steps, warmup, sweep, fused_only, rounds=5):
+    """-> dict with per-launch milliseconds of native A, native B, back-to-back and the fused kernel.
+
+    The four modes are timed in `rounds` interleaved rounds of steps/rounds launches each and the
+    median round is reported, so slow drifts of clocks hit all modes alike."""
+    import statistics
     plans = candidate_plans(cfg, pair.k1, pair.k2, sweep)
-    base = plans[0][1]
+    plan, label = plans[0][1], plans[0][0]
+    if len(plans) > 1:
+        best = None
+        probe = max(20, steps // 4)
+        for lab, p in plans:
+            t = p.time(3, pair.args1, pair.args2, max(5, warmup // 2), probe) / probe
+            if best is None or t < best[0]:
+                best = (t, lab, p)
+        _, label, plan = best
+    per = max(1, steps // rounds)
+    modes = [3] if fused_only else [0, 1, 2, 3]
+    samples = {m: [] for m in modes}
+    for r in range(rounds):
+        for m in modes:
+            samples[m].append(plan.time(m, pair.args1, pair.args2, warmup if r == 0 else 2, per) / per)
     res = {}
-    if not fused_only:
-        res["t_a_ms"] = base.time(0, pair.args1, pair.args2, warmup, steps) / steps
-        res["t_b_ms"] = base.time(1, pair.args1, pair.args2, warmup, steps) / steps
-        res["t_b2b_ms"] = base.time(2, pair.args1, pair.args2, warmup, steps) / steps
-    best = None
-    probe = max(20, steps // 4)
-    for label, plan in plans:
-        t = plan.time(3, pair.args1, pair.args2, max(5, warmup // 2), probe) / probe
-        if best is None or t < best[0]:
-            best = (t, label, plan)
-    _, label, plan = best
-    res["t_fused_ms"] = plan.time(3, pair.args1, pair.args2, warmup, steps) / steps
+    names = {0: "t_a_ms", 1: "t_b_ms", 2: "t_b2b_ms", 3: "t_fused_ms"}
+    for m in modes:
+        res[names[m]] = statistics.median(samples[m])
     res["split"] = label
     part = plan.partition
     res["fused_name"] = part.name.decode()

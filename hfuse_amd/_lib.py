@@ -126,6 +126,8 @@ PROTOTYPES = {
     "hf_plan_free": (None, [C.c_void_p]),
     "hf_plan_set_barrier_mode": (C.c_int, [C.c_void_p, C.c_int]),
     "hf_plan_set_grids": (C.c_int, [C.c_void_p, C.c_int, C.c_int]),
+    "hf_plan_set_lending": (C.c_int, [C.c_void_p, C.c_int]),
+    "hf_plan_set_block": (C.c_int, [C.c_void_p, C.c_int, C.c_int]),
     "hf_plan_partition": (C.c_int, [C.c_void_p, C.POINTER(Partition)]),
     "hf_plan_num_splits": (C.c_int, [C.c_void_p, C.c_int]),
     "hf_plan_local_index": (C.c_int, [C.c_void_p, C.c_int, C.c_uint32, C.POINTER(Dim3)]),

@@ -66,6 +66,9 @@ bool lookup_kernel(const std::string &name, KernelId &id) {
 // reference as well: BarrierRewriter rewrites whatever __syncthreads it finds).
 bool body_has_barriers(KernelId id) { return id == K_BNSTATS || id == K_HISTC; }
 
+// Bodies that walk one flat index range (K::kFlat): they can run on a partner's idle waves.
+bool body_is_flat(KernelId id) { return id != K_BNSTATS && id != K_HISTC && id != K_ETHASH; }
+
 // ------------------------------------------------ constants of the searches
 struct SearchConstants {
   std::mutex mu;
@@ -338,7 +341,7 @@ unsigned long long wanted_blocks(const Prepared &p, unsigned threads) {
 }
 
 // Default grid of one kernel inside a block of `block_threads` threads: enough workgroups
-// to fill every CU eight times over, never more than the work asks for.  The streaming
+// to fill every CU sixteen times over, never more than the work asks for.  The streaming
 // bodies stride over the rest; a larger grid evens out their tail.  The histogram is the
 // exception: every block flushes its LDS bins with one global atomic per bin, so it runs
 // one block per CU and keeps eight loads per lane in flight instead.
@@ -348,7 +351,7 @@ unsigned default_grid(const Prepared &p, unsigned own_threads, unsigned block_th
   // (two per CU when it shares its blocks with a partner that ends early)
   const unsigned long long cap = p.id == K_HISTC
                                      ? (unsigned long long)cu_count() * (own_threads == block_threads ? 1u : 2u)
-                                     : (unsigned long long)cu_count() * per_cu * 8ull;
+                                     : (unsigned long long)cu_count() * per_cu * 16ull;
   return (unsigned)std::min(std::max(want, 1ull), cap);
 }
 
@@ -382,6 +385,7 @@ struct hf_plan {
   Partition part;
   int barrier_mode;
   unsigned grid_override[2] = {0, 0};  // hf_plan_set_grids
+  bool lending = true;                 // hf_plan_set_lending
 };
 
 // ------------------------------------------------------------------ C-ABI
@@ -491,6 +495,14 @@ HF_API int hf_plan_create(const hf_config *cfg, int fusion_index, const char *pr
     delete plan;
     return fail(rc, err);
   }
+  if (split_idx == HF_SPLIT_TABLE && f.threads > 0 && !p->base_line && (uint32_t)split_threads == f.split) {
+    // the pair's tuned block shape from the fusion list: Split threads of kernel 1 in a block of Threads
+    rc = hf_plan_set_block(plan, (int)f.split, (int)(f.threads - f.split));
+    if (rc != HF_OK) {
+      delete plan;
+      return rc;
+    }
+  }
   if (is_crypto(plan->ids[0]) && !p->base_line && plan->part.launch_threads > 512) {
     delete plan;
     return fail(HF_EINVAL, "search kernels are built for fused blocks of at most 512 threads");
@@ -532,6 +544,37 @@ HF_API int hf_plan_set_grids(hf_plan *plan, int grid1, int grid2) {
   if (grid1 < 0 || grid2 < 0) return fail(HF_EINVAL, "negative grid");
   plan->grid_override[0] = (unsigned)grid1;
   plan->grid_override[1] = (unsigned)grid2;
+  return HF_OK;
+}
+
+HF_API int hf_plan_set_block(hf_plan *plan, int threads1, int threads2) {
+  if (!plan) return fail(HF_EINVAL, "null plan");
+  if (plan->preset->base_line) return fail(HF_EINVAL, "vertical presets have no thread partition to set");
+  if (threads1 <= 0 || threads2 <= 0 || threads1 % (int)kWave || threads2 % (int)kWave)
+    return fail(HF_EINVAL, "both parts must be positive multiples of the 64-lane wavefront");
+  // Same rule as the re-split of the reference's Context (KernelFusion.h:72): BlockDim.X = threads / BlockDim.Y.
+  KernelRow rows[2] = {plan->rows[0], plan->rows[1]};
+  const int want[2] = {threads1, threads2};
+  for (int i = 0; i < 2; i++) {
+    if (rows[i].block_dim.z != 1 || want[i] % (int)rows[i].block_dim.y)
+      return fail(HF_EINVAL, "thread count does not divide by BlockDim.Y of '" + rows[i].name + "'");
+    rows[i].block_dim.x = (uint32_t)want[i] / rows[i].block_dim.y;
+  }
+  if (is_crypto(plan->ids[0]) && threads1 + threads2 > 512)
+    return fail(HF_EINVAL, "search kernels are built for fused blocks of at most 512 threads");
+  Partition part;
+  std::string err;
+  int rc = make_partition(rows[0], rows[1], *plan->preset, HF_SPLIT_TABLE, 0, part, err);
+  if (rc != HF_OK) return fail(rc, err);
+  part.name = plan->rows[0].name + "_" + plan->rows[1].name + "_fused_kernel_" + plan->preset->name + "_block_" +
+              std::to_string(threads1) + "_" + std::to_string(threads2);
+  plan->part = part;
+  return HF_OK;
+}
+
+HF_API int hf_plan_set_lending(hf_plan *plan, int on) {
+  if (!plan) return fail(HF_EINVAL, "null plan");
+  plan->lending = on != 0;
   return HF_OK;
 }
 
@@ -634,6 +677,7 @@ int do_launch_fused(const hf_plan *plan, const Prepared &p1, const Prepared &p2,
   g.hint1 = p1.hint;
   g.hint2 = p2.hint;
   g.grid1 = g.grid2 = 0;
+  g.lend = 0;
   const bool crypto = is_crypto(plan->ids[0]);
   const unsigned exact = grid_blocks > 0 ? (unsigned)grid_blocks : kDefaultEthashGrid;
   hipError_t e;
@@ -661,6 +705,16 @@ int do_launch_fused(const hf_plan *plan, const Prepared &p1, const Prepared &p2,
       g.grid2 = p2.exact_grid ? exact : default_grid(p2, g.d2, block);
       if (plan->grid_override[0] && !p1.exact_grid) g.grid1 = plan->grid_override[0];
       if (plan->grid_override[1] && !p2.exact_grid) g.grid2 = plan->grid_override[1];
+    }
+    // Wave lending: in the blocks only one kernel strides over, the other half's waves run
+    // that kernel too, so those blocks are d1+d2 threads wide for it and it needs fewer of them.
+    g.lend = plan->lending && grid_blocks <= 0;
+    if (g.lend) {
+      const unsigned dd = g.d1 + g.d2;
+      if (g.grid2 > g.grid1 && body_is_flat(plan->ids[1]) && !p2.exact_grid)
+        g.grid2 = g.grid1 + (unsigned)(((unsigned long long)(g.grid2 - g.grid1) * g.d2 + dd - 1) / dd);
+      else if (g.grid1 > g.grid2 && body_is_flat(plan->ids[0]) && !p1.exact_grid)
+        g.grid1 = g.grid2 + (unsigned)(((unsigned long long)(g.grid1 - g.grid2) * g.d1 + dd - 1) / dd);
     }
     const unsigned grid = std::max(g.grid1, g.grid2);
     const size_t lds = 4 * kBarrierWords + g.lds1 + g.lds2;

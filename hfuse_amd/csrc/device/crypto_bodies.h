@@ -95,11 +95,12 @@ __device__ __forceinline__ void sha256_compress(u32 st[8], u32 w[16]) {
 struct Sha256dBody {
   using Args = Sha256dDevArgs;
   static constexpr bool kBarriers = false;
+  static constexpr bool kFlat = true;
 
   template <class SB>
   static __device__ void run(const Args &a, SB &sb, unsigned char *, unsigned) {
-    const u32 stride = sb.nblocks * sb.nthreads;
-    for (u32 t = sb.bid * sb.nthreads + sb.tid; t < a.threads; t += stride) {
+    const u32 stride = sb.gstride();
+    for (u32 t = sb.gtid(); t < a.threads; t += stride) {
       const u32 nonce = a.start_nonce + t;
       u32 st[8], w[16];
 #pragma unroll
@@ -220,11 +221,12 @@ template <int NONCE_WORD, bool NONCE_HIGH>
 struct Blake2bBody {
   using Args = Blake2bDevArgs;
   static constexpr bool kBarriers = false;
+  static constexpr bool kFlat = true;
 
   template <class SB>
   static __device__ void run(const Args &a, SB &sb, unsigned char *, unsigned) {
-    const u32 stride = sb.nblocks * sb.nthreads;
-    for (u32 t = sb.bid * sb.nthreads + sb.tid; t < a.threads; t += stride) {
+    const u32 stride = sb.gstride();
+    for (u32 t = sb.gtid(); t < a.threads; t += stride) {
       const u32 nonce = a.start_nonce + t;
       u64 m[16], v[16];
 #pragma unroll
@@ -313,6 +315,7 @@ __device__ __forceinline__ u32 fnv_reduce(u32x4 v) { return fnv(fnv(fnv(v.x, v.y
 struct EthashBody {
   using Args = EthashDevArgs;
   static constexpr bool kBarriers = false;
+  static constexpr bool kFlat = false;  // one nonce per thread of the launch grid
   static constexpr int kGroup = 8, kParallel = 4, kAccesses = 64;
 
   template <class SB>

@@ -35,6 +35,7 @@ __device__ __forceinline__ void st4(float *p, f32x4 v) {
 struct Im2colBody {
   using Args = hf_im2col_args;
   static constexpr bool kBarriers = false;
+  static constexpr bool kFlat = true;  // walks one flat index range: may borrow a partner's idle waves
 
   template <class SB>
   static __device__ void run(const Args &a, SB &sb, unsigned char *, unsigned hint) {
@@ -42,9 +43,9 @@ struct Im2colBody {
       vec4_3x3(a, sb);
       return;
     }
-    const int64_t stride = (int64_t)sb.nblocks * sb.nthreads;
+    const int64_t stride = (int64_t)sb.gstride();
     const int64_t plane_col = a.height_col * a.width_col;
-    for (int64_t index = (int64_t)sb.bid * sb.nthreads + sb.tid; index < a.n; index += stride) {
+    for (int64_t index = (int64_t)sb.gtid(); index < a.n; index += stride) {
       const int64_t w_out = index % a.width_col;
       const int64_t idx = index / a.width_col;
       const int64_t h_out = idx % a.height_col;
@@ -76,8 +77,8 @@ struct Im2colBody {
     const unsigned wq = W >> 2;
     const unsigned plane = H * W;
     const unsigned n4 = (unsigned)(a.n >> 2);
-    const unsigned stride = sb.nblocks * sb.nthreads;
-    for (unsigned idx4 = sb.bid * sb.nthreads + sb.tid; idx4 < n4; idx4 += stride) {
+    const unsigned stride = sb.gstride();
+    for (unsigned idx4 = sb.gtid(); idx4 < n4; idx4 += stride) {
       const unsigned w4 = idx4 % wq;
       const unsigned t = idx4 / wq;
       const unsigned h_out = t % H;
@@ -119,13 +120,14 @@ struct Im2colBody {
 struct MaxPoolBody {
   using Args = hf_maxpool_args;
   static constexpr bool kBarriers = false;
+  static constexpr bool kFlat = true;
 
   template <class SB>
   static __device__ void run(const Args &a, SB &sb, unsigned char *, unsigned hint) {
     if (hint == HINT_POOL_K3S2P1) { vec2_s2<3, 1>(a, sb); return; }
     if (hint == HINT_POOL_K2S2P0) { vec2_s2<2, 0>(a, sb); return; }
-    const int64_t stride = (int64_t)sb.nblocks * sb.nthreads;
-    for (int64_t index = (int64_t)sb.bid * sb.nthreads + sb.tid; index < a.nthreads; index += stride) {
+    const int64_t stride = (int64_t)sb.gstride();
+    for (int64_t index = (int64_t)sb.gtid(); index < a.nthreads; index += stride) {
       const int pw = (int)(index % a.pooled_width);
       const int ph = (int)((index / a.pooled_width) % a.pooled_height);
       const int c = (int)((index / a.pooled_width / a.pooled_height) % a.channels);
@@ -164,8 +166,8 @@ struct MaxPoolBody {
     const unsigned PW = (unsigned)a.pooled_width, PH = (unsigned)a.pooled_height;
     const unsigned ph2 = PW >> 1;
     const unsigned n2 = (unsigned)a.nthreads >> 1;
-    const unsigned stride = sb.nblocks * sb.nthreads;
-    for (unsigned idx2 = sb.bid * sb.nthreads + sb.tid; idx2 < n2; idx2 += stride) {
+    const unsigned stride = sb.gstride();
+    for (unsigned idx2 = sb.gtid(); idx2 < n2; idx2 += stride) {
       const unsigned pw2 = idx2 % ph2;
       const unsigned t = idx2 / ph2;
       const unsigned ph = t % PH;
@@ -239,6 +241,7 @@ struct MaxPoolBody {
 struct UpsampleNearestBody {
   using Args = hf_upsample_nearest_args;
   static constexpr bool kBarriers = false;
+  static constexpr bool kFlat = true;
 
   template <class SB>
   static __device__ void run(const Args &a, SB &sb, unsigned char *, unsigned hint) {
@@ -250,9 +253,9 @@ struct UpsampleNearestBody {
       const unsigned w1h = (unsigned)a.width1 >> 1;
       const unsigned w2 = (unsigned)a.width2;
       const unsigned n2 = (unsigned)(a.nc * a.height1) * w1h;
-      const unsigned stride = sb.nblocks * sb.nthreads;
+      const unsigned stride = sb.gstride();
       const f32x2 *in = reinterpret_cast<const f32x2 *>(a.idata);
-      for (unsigned idx = sb.bid * sb.nthreads + sb.tid; idx < n2; idx += 2 * stride) {
+      for (unsigned idx = sb.gtid(); idx < n2; idx += 2 * stride) {
         const unsigned idx_b = idx + stride;
         const bool has_b = idx_b < n2;
         const f32x2 va = in[idx];
@@ -275,8 +278,8 @@ struct UpsampleNearestBody {
       return;
     }
     const size_t total = a.nc * a.height2 * a.width2;
-    const size_t stride = (size_t)sb.nblocks * sb.nthreads;
-    for (size_t index = (size_t)sb.bid * sb.nthreads + sb.tid; index < total; index += stride) {
+    const size_t stride = (size_t)sb.gstride();
+    for (size_t index = (size_t)sb.gtid(); index < total; index += stride) {
       const size_t x2 = index % a.width2;
       const size_t y2 = (index / a.width2) % a.height2;
       const size_t c = index / a.width2 / a.height2;
@@ -334,6 +337,7 @@ __device__ __forceinline__ Welford wave_merge(Welford w) {
 struct BnStatsBody {
   using Args = hf_bn_stats_args;
   static constexpr bool kBarriers = true;
+  static constexpr bool kFlat = false;  // one plane per block: the block index is part of the work mapping
   static constexpr unsigned kLdsBytes = 16 * sizeof(Welford) + 16;
 
   template <class SB>
@@ -410,6 +414,7 @@ struct BnStatsBody {
 struct HistcBody {
   using Args = hf_histc_args;
   static constexpr bool kBarriers = true;
+  static constexpr bool kFlat = false;  // block-private LDS bins
 
   // bin = (int)((v - min) * nbins / (max - min)) in fp32, bin == nbins -> nbins - 1.
   // POW2: max - min is a power of two, so the correctly rounded division equals the
@@ -449,8 +454,8 @@ struct HistcBody {
     };
     if (hint & HINT_HIST_VEC4) {
       const int64_t n4 = total >> 2;
-      const int64_t stride = (int64_t)sb.nblocks * sb.nthreads;
-      int64_t i = (int64_t)sb.bid * sb.nthreads + sb.tid;
+      const int64_t stride = (int64_t)sb.gstride();
+      int64_t i = (int64_t)sb.gtid();
       // several 16-byte loads in flight per lane before the dependent LDS atomics
 #ifndef HF_HIST_U
 #define HF_HIST_U 8
@@ -467,9 +472,9 @@ struct HistcBody {
         for (int64_t k = (n4 << 2) + sb.tid; k < total; k += sb.nthreads)
           count<POW2>(bins, b[k], lo, hi, fn, range, inv_range, nbins);
     } else {
-      const int64_t stride = (int64_t)sb.nblocks * sb.nthreads;
+      const int64_t stride = (int64_t)sb.gstride();
       const int64_t bs = a.b.strides[0];
-      for (int64_t i = (int64_t)sb.bid * sb.nthreads + sb.tid; i < total; i += stride)
+      for (int64_t i = (int64_t)sb.gtid(); i < total; i += stride)
         count<POW2>(bins, b[i * bs], lo, hi, fn, range, inv_range, nbins);
     }
     sb.sync();

@@ -37,6 +37,14 @@ struct SubBlock {
   unsigned nblocks;   // grid size the body strides by
   unsigned *bar;      // LDS arrival counter of this half (BAR_SUBSET only)
   unsigned phase;     // barriers this thread has passed
+  unsigned gbase;     // index of this half's thread 0 among all threads that run this kernel
+  unsigned gthreads;  // number of threads that run this kernel in the whole launch
+
+  // Flat work-item index and stride of a body that walks a 1-D range.  Equal to
+  // bid * nthreads + tid and nblocks * nthreads except where a block lends the idle
+  // half's waves to the partner (see fused_kernel), which makes blocks unequal in size.
+  __device__ __forceinline__ unsigned gtid() const { return gbase + tid; }
+  __device__ __forceinline__ unsigned gstride() const { return gthreads; }
 
   __device__ __forceinline__ unsigned lane() const { return tid & 63u; }
   __device__ __forceinline__ unsigned wave() const { return tid >> 6; }
@@ -67,6 +75,7 @@ struct FuseGeom {
   unsigned hint1, hint2;    // fast-path selector the host derived from each argument list
   unsigned grid1, grid2;    // workgroups each kernel strides over: in the fused kernel half k works in
                             // blocks [0, grid_k) only; in blockIdx mode kernel 2 starts at block grid1
+  unsigned lend;            // 1: in a block beyond its own grid a half's waves run the partner's body
 };
 
 constexpr unsigned kBarrierWords = 4;  // 16 bytes reserved at the base of LDS for arrival counters
@@ -75,7 +84,8 @@ constexpr unsigned kBarrierWords = 4;  // 16 bytes reserved at the base of LDS f
 template <class K, int T>
 __global__ __launch_bounds__(T) void native_kernel(typename K::Args a, unsigned hint) {
   extern __shared__ __align__(16) unsigned char smem[];
-  SubBlock<BAR_WORKGROUP> sb{threadIdx.x, blockDim.x, blockIdx.x, gridDim.x, nullptr, 0};
+  SubBlock<BAR_WORKGROUP> sb{threadIdx.x, blockDim.x, blockIdx.x, gridDim.x, nullptr, 0,
+                             blockIdx.x * blockDim.x, gridDim.x * blockDim.x};
   K::run(a, sb, smem, hint);
 }
 
@@ -98,16 +108,42 @@ __global__ __launch_bounds__(T) void fused_kernel(typename K1::Args a1, typename
   constexpr int B1 = (kSubset && K1::kBarriers) ? BAR_SUBSET : BAR_WORKGROUP;
   constexpr int B2 = (kSubset && K2::kBarriers) ? BAR_SUBSET : BAR_WORKGROUP;
   // Both halves see the launch's blockIdx (the reference leaves blockIdx/gridDim alone,
-  // include/ThreadInfoRewriter.h:29-31); a half whose kernel wants fewer workgroups than the
-  // launch has simply ends in the surplus blocks, which frees its wave slots for the partner.
-  if (wave < (g.d1 >> 6)) {
-    if (blockIdx.x >= g.grid1) return;
-    SubBlock<B1> sb{tid, g.d1, blockIdx.x, g.grid1, bars + 0, 0};
-    K1::run(a1, sb, smem + 4 * kBarrierWords, g.hint1);
-  } else {
-    if (blockIdx.x >= g.grid2) return;
-    SubBlock<B2> sb{tid - g.d1, g.d2, blockIdx.x, g.grid2, bars + 1, 0};
-    K2::run(a2, sb, smem + 4 * kBarrierWords + g.lds1, g.hint2);
+  // include/ThreadInfoRewriter.h:29-31).  A half whose kernel wants fewer workgroups than the
+  // launch has would idle in the surplus blocks; there its waves either end at once (freeing
+  // their slots) or, when the partner walks a flat 1-D range (K::kFlat) and lending is on,
+  // run the partner's body, so a surplus block is one whole block of the partner.  The
+  // partner's flat index then counts d_partner threads in shared blocks and d1+d2 in lent ones.
+  const unsigned bid = blockIdx.x, dd = g.d1 + g.d2;
+  const bool in1 = bid < g.grid1, in2 = bid < g.grid2;
+  const bool lend1 = K1::kFlat && g.lend && g.grid1 > g.grid2;  // kernel 1 borrows kernel 2's waves
+  const bool lend2 = K2::kFlat && g.lend && g.grid2 > g.grid1;  // kernel 2 borrows kernel 1's waves
+  const unsigned total1 = lend1 ? g.grid2 * g.d1 + (g.grid1 - g.grid2) * dd : g.grid1 * g.d1;
+  const unsigned total2 = lend2 ? g.grid1 * g.d2 + (g.grid2 - g.grid1) * dd : g.grid2 * g.d2;
+  unsigned char *lds1 = smem + 4 * kBarrierWords, *lds2 = lds1 + g.lds1;
+  if (in1 && in2) {  // a shared block
+    if (wave < (g.d1 >> 6)) {
+      SubBlock<B1> sb{tid, g.d1, bid, g.grid1, bars + 0, 0, bid * g.d1, total1};
+      K1::run(a1, sb, lds1, g.hint1);
+    } else {
+      SubBlock<B2> sb{tid - g.d1, g.d2, bid, g.grid2, bars + 1, 0, bid * g.d2, total2};
+      K2::run(a2, sb, lds2, g.hint2);
+    }
+  } else if (in1) {  // kernel 2 has no work here
+    if (lend1) {
+      SubBlock<BAR_WORKGROUP> sb{tid, dd, bid, g.grid1, nullptr, 0, g.grid2 * g.d1 + (bid - g.grid2) * dd, total1};
+      K1::run(a1, sb, lds1, g.hint1);
+    } else if (wave < (g.d1 >> 6)) {
+      SubBlock<B1> sb{tid, g.d1, bid, g.grid1, bars + 0, 0, bid * g.d1, total1};
+      K1::run(a1, sb, lds1, g.hint1);
+    }
+  } else if (in2) {  // kernel 1 has no work here
+    if (lend2) {
+      SubBlock<BAR_WORKGROUP> sb{tid, dd, bid, g.grid2, nullptr, 0, g.grid1 * g.d2 + (bid - g.grid1) * dd, total2};
+      K2::run(a2, sb, lds2, g.hint2);
+    } else if (wave >= (g.d1 >> 6)) {
+      SubBlock<B2> sb{tid - g.d1, g.d2, bid, g.grid2, bars + 1, 0, bid * g.d2, total2};
+      K2::run(a2, sb, lds2, g.hint2);
+    }
   }
 }
 
@@ -121,11 +157,12 @@ __global__ __launch_bounds__(T) void blockidx_kernel(typename K1::Args a1, typen
   const unsigned tid = threadIdx.x;
   if (blockIdx.x < g.grid1) {
     if (tid >= g.d1) return;
-    SubBlock<BAR_WORKGROUP> sb{tid, g.d1, blockIdx.x, g.grid1, nullptr, 0};
+    SubBlock<BAR_WORKGROUP> sb{tid, g.d1, blockIdx.x, g.grid1, nullptr, 0, blockIdx.x * g.d1, g.grid1 * g.d1};
     K1::run(a1, sb, smem, g.hint1);
   } else {
     if (tid >= g.d2) return;
-    SubBlock<BAR_WORKGROUP> sb{tid, g.d2, blockIdx.x - g.grid1, g.grid2, nullptr, 0};
+    const unsigned b2 = blockIdx.x - g.grid1;
+    SubBlock<BAR_WORKGROUP> sb{tid, g.d2, b2, g.grid2, nullptr, 0, b2 * g.d2, g.grid2 * g.d2};
     K2::run(a2, sb, smem, g.hint2);
   }
 }

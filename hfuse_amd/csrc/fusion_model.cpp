@@ -147,8 +147,15 @@ bool parse_config(const char *fusion_yaml, const char *kernels_yaml, Config &cfg
           return false;
         }
       }
+      if (const YamlNode *th = n.get("Threads")) {
+        if (!to_uint(th, f.threads) || f.threads % kWave != 0 || f.threads > kMaxBlock || f.split == 0 ||
+            f.threads <= f.split) {
+          err = "fusion list: " + at(*th) + "'Threads' must be a multiple of 64, at most 1024 and larger than 'Split'";
+          return false;
+        }
+      }
       for (auto &kv : n.map)
-        if (kv.first != "File" && kv.first != "Kernels" && kv.first != "Split") {
+        if (kv.first != "File" && kv.first != "Kernels" && kv.first != "Split" && kv.first != "Threads") {
           err = "fusion list: " + at(kv.second) + "unknown key '" + kv.first + "'";
           return false;
         }

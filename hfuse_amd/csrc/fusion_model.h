@@ -28,7 +28,8 @@ struct KernelRow {
 struct FusionRow {
   std::string file;
   std::vector<std::string> kernels;
-  uint32_t split = 0;  // optional `Split:` key: threads of kernel 1 when the caller asks for the table split
+  uint32_t split = 0;    // optional `Split:` key: threads of kernel 1 when the caller asks for the table split
+  uint32_t threads = 0;  // optional `Threads:` key: threads of the whole fused block (needs Split)
 };
 
 struct Config {

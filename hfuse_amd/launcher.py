@@ -109,6 +109,12 @@ class Plan:
     def set_grids(self, grid1: int = 0, grid2: int = 0) -> None:
         check(L.lib().hf_plan_set_grids(self._h, grid1, grid2))
 
+    def set_block(self, threads1: int, threads2: int) -> None:
+        check(L.lib().hf_plan_set_block(self._h, threads1, threads2))
+
+    def set_lending(self, on: bool) -> None:
+        check(L.lib().hf_plan_set_lending(self._h, int(on)))
+
     def local_index(self, half: int, tid: int):
         out = L.Dim3()
         check(L.lib().hf_plan_local_index(self._h, half, tid, C.byref(out)))

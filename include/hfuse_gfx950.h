@@ -75,9 +75,10 @@ typedef struct {
  * and a string-keyed map of kernel rows.  `kernels_yaml` may also be the older
  * per-pair form, a bare sequence of rows (configs/im2col_maxpool.yaml); then
  * `fusion_yaml` may be NULL and the single fusion is that list in order.
- * One key beyond the reference's schema is accepted in a fusion entry:
- * `Split: <threads>`, a tuned default for kernel 1's share of the block, used
- * when a plan is created with HF_SPLIT_TABLE.
+ * Two keys beyond the reference's schema are accepted in a fusion entry:
+ * `Split: <threads>`, a tuned default for kernel 1's share of the block, and
+ * `Threads: <threads>`, a tuned size of the whole fused block (kernel 2 gets
+ * Threads - Split); both apply when a plan is created with HF_SPLIT_TABLE.
  */
 HF_API int hf_config_load_text(const char *fusion_yaml, const char *kernels_yaml, hf_config **out);
 HF_API int hf_config_load_files(const char *fusion_path, const char *kernels_path, hf_config **out);
@@ -149,6 +150,22 @@ HF_API int hf_plan_set_barrier_mode(hf_plan *plan, int mode);
  * the surplus ones.)
  */
 HF_API int hf_plan_set_grids(hf_plan *plan, int grid1, int grid2);
+/*
+ * Give the fused block an explicit shape: threads1 for kernel 1 and threads2 for
+ * kernel 2 (multiples of 64, sum <= 1024), independent of the kernel table's
+ * BlockDim, which stays the native launch shape.  The reference reaches the same
+ * freedom through per-pair kernel tables (configs/im2col_maxpool.yaml ...).
+ */
+HF_API int hf_plan_set_block(hf_plan *plan, int threads1, int threads2);
+/*
+ * Wave lending (on by default).  When the two halves stride over different numbers
+ * of blocks, the blocks beyond the smaller grid have one half without work.  With
+ * lending on, that half's wavefronts run the partner's body there (the partner must
+ * walk a flat 1-D index range: im2col, max-pool, upsample, SHA-256d, Blake2b), so
+ * such a block is d1+d2 threads of the partner.  Off: the idle half's waves end at
+ * once, which is what the reference's generated kernel does.  Results are identical.
+ */
+HF_API int hf_plan_set_lending(hf_plan *plan, int on);
 HF_API int hf_plan_partition(const hf_plan *plan, hf_partition *out);
 /* Number of variants the reference's split loop would print (main.cpp:221-223). */
 HF_API int hf_plan_num_splits(const hf_config *cfg, int fusion_index);

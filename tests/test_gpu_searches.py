@@ -145,6 +145,24 @@ def test_fused_sha256d_sia(cuda, cfg):
         assert H.read_search_results(r2) == want2
 
 
+def test_fused_search_unequal_grids_with_and_without_lending(cuda, cfg):
+    h1, h2 = O.seeded_bytes(80, SEED + 21), O.seeded_bytes(80, SEED + 22)
+    H.sha256d_set_block(h1, EASY12)
+    H.sia_blake2b_set_block(h2)
+    want1 = oracle_hits(O.sha256d_search(h1, 0, 1 << 16, EASY12))
+    want2 = oracle_hits(O.sia_search(h2, 0, 1 << 17, EASY12))
+    plan = cfg.plan(cfg.find_fusion("sha256d_gpu_hash_shared", "sia_blake2b_gpu_hash"))
+    for lend in (True, False):
+        plan.set_lending(lend)
+        for grids in ((5, 40), (40, 5)):
+            plan.set_grids(*grids)
+            r1, r2 = H.new_search_results(), H.new_search_results()
+            plan.launch(H.sha256d_args(r1, 1 << 16, 0), H.blake2b_args(r2, 1 << 17, 0, EASY12))
+            sync()
+            assert H.read_search_results(r1) == want1
+            assert H.read_search_results(r2) == want2
+
+
 def test_fused_ethash_sia(cuda, cfg):
     n_items = 1 << 16
     dag = _dag(cuda, n_items, SEED)

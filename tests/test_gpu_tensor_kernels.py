@@ -298,6 +298,34 @@ def test_fused_histc_maxpool(cuda, cfg):
             b.check()
 
 
+@pytest.mark.parametrize("lend", [True, False])
+def test_wave_lending_gives_identical_results(cuda, cfg, lend):
+    """Blocks beyond one half's grid: with lending the idle half runs the partner's body,
+    without it those waves end at once; both must produce the same bits."""
+    cases = [
+        ("batch_norm_collect_statistics_kernel", "upsample_nearest2d_out_frame",
+         lambda: BnStats(cuda, 8, 5, 14, 14), lambda: Upsample(cuda, 8, 16, 28, 28, (56, 56))),
+        ("upsample_nearest2d_out_frame", "batch_norm_collect_statistics_kernel",
+         lambda: Upsample(cuda, 8, 16, 28, 28, (56, 56)), lambda: BnStats(cuda, 8, 5, 14, 14)),
+        ("kernelHistogram1D", "MaxPoolForward",
+         lambda: Histc(cuda, 30000), lambda: MaxPool(cuda, 8, 32, 64, 64, (2, 2), (2, 2), (0, 0))),
+        ("im2col_kernel", "MaxPoolForward",
+         lambda: Im2col(cuda, 1, 2, 8, 8), lambda: MaxPool(cuda, 8, 32, 64, 64, (3, 3), (2, 2), (1, 1))),
+        ("im2col_kernel", "MaxPoolForward",
+         lambda: Im2col(cuda, 8, 16, 56, 56), lambda: MaxPool(cuda, 1, 2, 8, 8, (2, 2), (2, 2), (0, 0))),
+    ]
+    for k1, k2, m1, m2 in cases:
+        plan = cfg.plan(cfg.find_fusion(k1, k2))
+        plan.set_lending(lend)
+        for grids in ((0, 0), (3, 11), (11, 3)):
+            plan.set_grids(*grids)
+            a, b = m1(), m2()
+            plan.launch(a.args, b.args)
+            sync()
+            a.check()
+            b.check()
+
+
 def test_fused_barrier_modes(cuda, cfg):
     """hist + bn both synchronise: subset counters, the shared hardware barrier and the
     blockIdx fallback must all give the same results."""
