@@ -16,6 +16,13 @@ namespace hfuse {
 enum { HINT_GENERIC = 0, HINT_IM2COL_3X3_S1P1 = 1, HINT_POOL_K3S2P1 = 1, HINT_POOL_K2S2P0 = 2, HINT_UP_2X = 1, HINT_BN_VEC4 = 1, HINT_HIST_VEC4 = 1, HINT_HIST_POW2 = 2 };
 
 __device__ __forceinline__ f32x4 ld4(const float *p) { return *reinterpret_cast<const f32x4 *>(p); }
+
+// One DPP move of a float.  0x138 = wave_shr:1 (lane i receives lane i-1's value),
+// 0x130 = wave_shl:1 (lane i receives lane i+1's); the lane without a source keeps 0.
+template <int CTRL>
+__device__ __forceinline__ float dpp_f32(float v) {
+  return __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), CTRL, 0xF, 0xF, false));
+}
 #ifndef HF_NT_STORES
 #define HF_NT_STORES 1
 #endif
@@ -69,8 +76,10 @@ struct Im2colBody {
 
   // 3x3, stride 1, pad 1, dilation 1, width % 4 == 0: a work item owns four
   // neighbouring output columns.  Per input row it needs columns w0-1 .. w0+4:
-  // one aligned 16-byte load plus the two edge scalars; each of the nine taps
-  // is then one 16-byte store.
+  // one aligned 16-byte load; the two edge columns are the neighbouring lanes'
+  // outer elements, moved with a wavefront-wide DPP shift (lanes 0 and 63 fetch
+  // theirs from memory).  Each of the nine taps is then one 16-byte store.  The
+  // trip count is wave-uniform so every lane's neighbour is live.
   template <class SB>
   static __device__ __forceinline__ void vec4_3x3(const Args &a, SB &sb) {
     const unsigned W = (unsigned)a.width, H = (unsigned)a.height;
@@ -78,7 +87,10 @@ struct Im2colBody {
     const unsigned plane = H * W;
     const unsigned n4 = (unsigned)(a.n >> 2);
     const unsigned stride = sb.gstride();
-    for (unsigned idx4 = sb.gtid(); idx4 < n4; idx4 += stride) {
+    const unsigned lane = sb.lane();
+    for (unsigned first = sb.gtid() - lane; first < n4; first += stride) {
+      const bool valid = first + lane < n4;
+      const unsigned idx4 = valid ? first + lane : n4 - 1;
       const unsigned w4 = idx4 % wq;
       const unsigned t = idx4 / wq;
       const unsigned h_out = t % H;
@@ -86,28 +98,32 @@ struct Im2colBody {
       const unsigned w0 = w4 << 2;
       const float *im = a.data_im + (size_t)c * plane;
       float *col = a.data_col + (size_t)c * 9u * plane + (size_t)h_out * W + w0;
+      const bool has_left = w0 > 0, has_right = w0 + 4 < W;
       float r[3][6];
 #pragma unroll
       for (int i = 0; i < 3; i++) {
         const int h = (int)h_out - 1 + i;
-        if (h >= 0 && h < (int)H) {
-          const float *row = im + (unsigned)h * W + w0;
-          const f32x4 m = ld4(row);
-          r[i][0] = w0 > 0 ? row[-1] : 0.0f;
-          r[i][1] = m.x; r[i][2] = m.y; r[i][3] = m.z; r[i][4] = m.w;
-          r[i][5] = (w0 + 4 < W) ? row[4] : 0.0f;
-        } else {
-#pragma unroll
-          for (int k = 0; k < 6; k++) r[i][k] = 0.0f;
-        }
+        const bool in = h >= 0 && h < (int)H;
+        const float *row = im + (unsigned)(in ? h : (int)h_out) * W + w0;
+        f32x4 m = ld4(row);
+        if (!in) m = f32x4{0.0f, 0.0f, 0.0f, 0.0f};
+        float left = dpp_f32<0x138>(m.w);   // wave_shr:1 -- lane-1's last column
+        float right = dpp_f32<0x130>(m.x);  // wave_shl:1 -- lane+1's first column
+        if (lane == 0 && has_left) left = in ? row[-1] : 0.0f;
+        if (lane == 63 && has_right) right = in ? row[4] : 0.0f;
+        r[i][0] = has_left ? left : 0.0f;
+        r[i][1] = m.x; r[i][2] = m.y; r[i][3] = m.z; r[i][4] = m.w;
+        r[i][5] = has_right ? right : 0.0f;
       }
+      if (valid) {
 #pragma unroll
-      for (int i = 0; i < 3; i++)
+        for (int i = 0; i < 3; i++)
 #pragma unroll
-        for (int j = 0; j < 3; j++) {
-          f32x4 v = {r[i][j], r[i][j + 1], r[i][j + 2], r[i][j + 3]};
-          st4(col + (size_t)(i * 3 + j) * plane, v);
-        }
+          for (int j = 0; j < 3; j++) {
+            f32x4 v = {r[i][j], r[i][j + 1], r[i][j + 2], r[i][j + 3]};
+            st4(col + (size_t)(i * 3 + j) * plane, v);
+          }
+      }
     }
   }
 };
