@@ -488,14 +488,16 @@ HF_API int hf_plan_create(const hf_config *cfg, int fusion_index, const char *pr
     return fail(HF_EUNSUPPORTED, "pairs mixing a tensor kernel with a search kernel are not built");
   }
   std::string err;
-  if (split_idx == HF_SPLIT_TABLE && split_threads <= 0 && f.split > 0 && !p->base_line)
-    split_threads = (int)f.split;  // the pair's tuned default from the fusion list
+  // The pair's tuned default from the fusion list: `Split` alone re-splits the table's block,
+  // `Split` + `Threads` give the fused block its own shape (applied below).
+  const bool tuned = split_idx == HF_SPLIT_TABLE && split_threads <= 0 && f.split > 0 && !p->base_line;
+  if (tuned && f.threads == 0) split_threads = (int)f.split;
   int rc = make_partition(plan->rows[0], plan->rows[1], *p, split_idx, split_threads, plan->part, err);
   if (rc != HF_OK) {
     delete plan;
     return fail(rc, err);
   }
-  if (split_idx == HF_SPLIT_TABLE && f.threads > 0 && !p->base_line && (uint32_t)split_threads == f.split) {
+  if (tuned && f.threads > 0) {
     // the pair's tuned block shape from the fusion list: Split threads of kernel 1 in a block of Threads
     rc = hf_plan_set_block(plan, (int)f.split, (int)(f.threads - f.split));
     if (rc != HF_OK) {

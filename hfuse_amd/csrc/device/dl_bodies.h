@@ -383,13 +383,16 @@ struct BnStatsBody {
           const unsigned b = ch / lq, q = ch - b * lq;
           return ld4(base + (size_t)b * a.input.strides[0] + (size_t)q * 4);
         };
+#ifndef HF_BN_U
+#define HF_BN_U 4
+#endif
         unsigned ch = sb.tid;
-        for (; ch + 3 * sb.nthreads < chunks; ch += 4 * sb.nthreads) {  // four loads in flight
-          f32x4 v[4];
+        for (; ch + (HF_BN_U - 1) * sb.nthreads < chunks; ch += HF_BN_U * sb.nthreads) {  // loads in flight
+          f32x4 v[HF_BN_U];
 #pragma unroll
-          for (int u = 0; u < 4; u++) v[u] = chunk(ch + u * sb.nthreads);
+          for (int u = 0; u < HF_BN_U; u++) v[u] = chunk(ch + u * sb.nthreads);
 #pragma unroll
-          for (int u = 0; u < 4; u++) merge4(v[u]);
+          for (int u = 0; u < HF_BN_U; u++) merge4(v[u]);
         }
         for (; ch < chunks; ch += sb.nthreads) merge4(chunk(ch));
         acc.n = 4.0f * k;

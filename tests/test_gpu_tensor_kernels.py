@@ -326,6 +326,28 @@ def test_wave_lending_gives_identical_results(cuda, cfg, lend):
             b.check()
 
 
+@pytest.mark.parametrize("block", [(64, 64), (128, 384), (512, 512), (256, 768), (960, 64)])
+def test_fused_block_shapes(cuda, cfg, block):
+    """Every legal shape of the fused block gives the same bits (all three benchmarked tensor pairs)."""
+    cases = [
+        ("im2col_kernel", "MaxPoolForward",
+         lambda: Im2col(cuda, 4, 16, 56, 56), lambda: MaxPool(cuda, 4, 16, 112, 112, (3, 3), (2, 2), (1, 1))),
+        ("batch_norm_collect_statistics_kernel", "upsample_nearest2d_out_frame",
+         lambda: BnStats(cuda, 16, 24, 28, 28), lambda: Upsample(cuda, 4, 16, 56, 56, (112, 112))),
+        ("kernelHistogram1D", "MaxPoolForward",
+         lambda: Histc(cuda, 1 << 21), lambda: MaxPool(cuda, 4, 32, 64, 64, (2, 2), (2, 2), (0, 0))),
+    ]
+    for k1, k2, m1, m2 in cases:
+        plan = cfg.plan(cfg.find_fusion(k1, k2))
+        plan.set_block(*block)
+        assert plan.partition.launch_threads == sum(block)
+        a, b = m1(), m2()
+        plan.launch(a.args, b.args)
+        sync()
+        a.check()
+        b.check()
+
+
 def test_fused_barrier_modes(cuda, cfg):
     """hist + bn both synchronise: subset counters, the shared hardware barrier and the
     blockIdx fallback must all give the same results."""

@@ -203,6 +203,44 @@ def test_split_rules():
     assert "1024" in e.value.message
 
 
+def test_tuned_split_and_block_keys_of_the_fusion_list():
+    """`Split` / `Threads` (beyond the reference's schema) give a pair its default fused block."""
+    fusion = ("- File: a\n  Split: 128\n  Kernels:\n    - im2col_kernel\n    - MaxPoolForward\n"
+              "- File: b\n  Split: 256\n  Threads: 512\n  Kernels:\n    - MaxPoolForward\n"
+              "    - batch_norm_collect_statistics_kernel\n")
+    cfg = Config(fusion, KERNELS_MAP)
+    a = cfg.plan(0).partition
+    assert (list(a.lo), list(a.hi)) == ([0, 128], [128, 768])        # re-split of the table's 512 + 256
+    b = cfg.plan(1).partition
+    assert (list(b.lo), list(b.hi), b.launch_threads) == ([0, 256], [256, 512], 512)
+    assert (b.block_dim[1].x, b.block_dim[1].y) == (16, 16)           # bn keeps Y, X = threads / Y
+    assert b.name == b"MaxPoolForward_batch_norm_collect_statistics_kernel_fused_kernel_hfuse_block_256_256"
+    # an explicit split index still follows the reference's enumeration over the table's block
+    assert list(cfg.plan(1, "hfuse", 0).partition.hi) == [128, 768]
+    for bad in ("  Split: 100\n", "  Split: 0\n", "  Split: 128\n  Threads: 128\n", "  Threads: 512\n",
+                "  Split: 128\n  Threads: 2048\n", "  Bogus: 1\n"):
+        with pytest.raises(hfuse_amd.HfuseError) as e:
+            Config("- File: a\n" + bad + "  Kernels:\n    - im2col_kernel\n    - MaxPoolForward\n", KERNELS_MAP)
+        assert e.value.code == L.HF_EPARSE
+
+
+def test_set_block_rules():
+    cfg = Config(FUSION, KERNELS_MAP)
+    plan = cfg.plan(1)  # MaxPool (256) + bn (32,16)
+    plan.set_block(128, 256)
+    p = plan.partition
+    assert (list(p.hi), p.block_dim[1].x, p.block_dim[1].y, p.launch_threads) == ([128, 384], 16, 16, 384)
+    for bad in ((100, 256), (0, 256), (128, 0), (512, 768), (128, 64 * 3 + 8)):
+        with pytest.raises(hfuse_amd.HfuseError):
+            plan.set_block(*bad)
+    with pytest.raises(hfuse_amd.HfuseError):
+        cfg.plan(1, "vfuse").set_block(128, 128)
+    plan.set_grids(3, 5)
+    plan.set_lending(False)
+    with pytest.raises(hfuse_amd.HfuseError):
+        plan.set_grids(-1, 0)
+
+
 def test_local_index_follows_the_remap(cfg):
     plan = cfg.plan(cfg.find_fusion("upsample_nearest2d_out_frame", "batch_norm_collect_statistics_kernel"))
     part = plan.partition
