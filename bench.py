@@ -168,6 +168,11 @@ def time_tensor_pair(cfg, pair, steps, warmup, sweep, fused_only, rounds=5):
     names = {0: "t_a_ms", 1: "t_b_ms", 2: "t_b2b_ms", 3: "t_fused_ms"}
     for m in modes:
         res[names[m]] = statistics.median(samples[m])
+    if not fused_only:
+        # the reference's vertical baseline (same threads run both bodies), for the three-way comparison
+        vplan = cfg.plan(cfg.find_fusion(pair.k1, pair.k2), "vfuse")
+        res["t_vfuse_ms"] = statistics.median(
+            [vplan.time(3, pair.args1, pair.args2, 2, per) / per for _ in range(3)])
     res["split"] = label
     part = plan.partition
     res["fused_name"] = part.name.decode()
@@ -236,6 +241,8 @@ def run_search_pair(cfg, name, log2_a, log2_b, sweep, fused_only, iters=2):
             best = (t, label, plan)
     _, label, plan = best
     res["t_fused_ms"] = plan.time(3, [a1], [a2], 0, iters, grid) / iters
+    if not fused_only:
+        res["t_vfuse_ms"] = cfg.plan(cfg.find_fusion(k1, k2), "vfuse").time(3, [a1], [a2], 0, 1, grid)
     res["split"] = label
     part = plan.partition
     res["fused_name"] = part.name.decode()

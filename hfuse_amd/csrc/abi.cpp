@@ -669,8 +669,6 @@ HF_API int hf_launch_native(const char *kernel_name, const void *args, int grid_
 namespace {
 
 int do_launch_fused(const hf_plan *plan, const Prepared &p1, const Prepared &p2, int grid_blocks, hipStream_t stream) {
-  if (plan->preset->base_line)
-    return fail(HF_EUNSUPPORTED, "vertical presets only report their partition; launch an hfuse preset");
   FuseGeom g;
   g.d1 = plan->part.hi[0] - plan->part.lo[0];
   g.d2 = plan->part.hi[1] - plan->part.lo[1];
@@ -683,7 +681,16 @@ int do_launch_fused(const hf_plan *plan, const Prepared &p1, const Prepared &p2,
   const bool crypto = is_crypto(plan->ids[0]);
   const unsigned exact = grid_blocks > 0 ? (unsigned)grid_blocks : kDefaultEthashGrid;
   hipError_t e;
-  if (plan->barrier_mode == HF_BARRIER_BLOCKIDX) {
+  if (plan->preset->base_line) {
+    // Vertical baseline: both kernels start at thread 0 of a block of max(d1, d2) threads.
+    const unsigned block = std::max(g.d1, g.d2);
+    g.grid1 = p1.exact_grid ? exact : (grid_blocks > 0 ? (unsigned)grid_blocks : default_grid(p1, g.d1, block));
+    g.grid2 = p2.exact_grid ? exact : (grid_blocks > 0 ? (unsigned)grid_blocks : default_grid(p2, g.d2, block));
+    const size_t lds = 4 * kBarrierWords + g.lds1 + g.lds2;
+    const unsigned grid = std::max(g.grid1, g.grid2);
+    e = crypto ? launch_fused_crypto(plan->ids[0], plan->ids[1], MODE_VERTICAL, p1.blob, p2.blob, g, grid, lds, stream)
+               : launch_fused_dl(plan->ids[0], plan->ids[1], MODE_VERTICAL, p1.blob, p2.blob, g, grid, lds, stream);
+  } else if (plan->barrier_mode == HF_BARRIER_BLOCKIDX) {
     // Each kernel gets its own workgroups inside one launch.
     const unsigned block = std::max(g.d1, g.d2);
     g.grid1 = p1.exact_grid ? exact : default_grid(p1, g.d1, block);

@@ -167,4 +167,31 @@ __global__ __launch_bounds__(T) void blockidx_kernel(typename K1::Args a1, typen
   }
 }
 
+// Vertical fusion, the reference's baseline presets (vfuse, vfuse_lb: main.cpp:183-184,
+// KernelFusion.h:76-78 -- both kernels start at thread 0): the block is max(d1, d2) threads
+// and the same threads run kernel 1's body and then kernel 2's.  A body that synchronises
+// uses its LDS arrival counter, because the threads beyond its own size are still alive
+// (they wait for, or already run, the other body) and must not be waited for.
+template <class K1, class K2, int T>
+__global__ __launch_bounds__(T) void vertical_kernel(typename K1::Args a1, typename K2::Args a2, FuseGeom g) {
+  extern __shared__ __align__(16) unsigned char smem[];
+  unsigned *bars = reinterpret_cast<unsigned *>(smem);
+  const unsigned tid = threadIdx.x, bid = blockIdx.x;
+  if constexpr (K1::kBarriers || K2::kBarriers) {
+    if (tid < kBarrierWords) bars[tid] = 0;
+    __syncthreads();
+  }
+  constexpr int B1 = K1::kBarriers ? BAR_SUBSET : BAR_WORKGROUP;
+  constexpr int B2 = K2::kBarriers ? BAR_SUBSET : BAR_WORKGROUP;
+  const unsigned wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  if (wave < (g.d1 >> 6) && bid < g.grid1) {
+    SubBlock<B1> sb{tid, g.d1, bid, g.grid1, bars + 0, 0, bid * g.d1, g.grid1 * g.d1};
+    K1::run(a1, sb, smem + 4 * kBarrierWords, g.hint1);
+  }
+  if (wave < (g.d2 >> 6) && bid < g.grid2) {
+    SubBlock<B2> sb{tid, g.d2, bid, g.grid2, bars + 1, 0, bid * g.d2, g.grid2 * g.d2};
+    K2::run(a2, sb, smem + 4 * kBarrierWords + g.lds1, g.hint2);
+  }
+}
+
 }  // namespace hfuse

@@ -31,6 +31,9 @@ hipError_t pair(FuseMode mode, const void *a1, const void *a2, const FuseGeom &g
       break;
     case MODE_MATCHED:
       return hipErrorNotSupported;  // none of the searches has a barrier
+    case MODE_VERTICAL:
+      hipLaunchKernelGGL((vertical_kernel<K1, K2, kCryptoBlock>), dim3(grid), dim3(g.d1 > g.d2 ? g.d1 : g.d2), lds, s, x1, x2, g);
+      break;
     case MODE_BLOCKIDX:
       hipLaunchKernelGGL((blockidx_kernel<K1, K2, kCryptoBlock>), dim3(grid), dim3(g.d1 > g.d2 ? g.d1 : g.d2), lds,
                          s, x1, x2, g);

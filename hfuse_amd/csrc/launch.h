@@ -21,7 +21,7 @@ enum KernelId {
   K_COUNT
 };
 
-enum FuseMode { MODE_HFUSE = 0, MODE_MATCHED = 1, MODE_BLOCKIDX = 2 };
+enum FuseMode { MODE_HFUSE = 0, MODE_MATCHED = 1, MODE_BLOCKIDX = 2, MODE_VERTICAL = 3 };
 
 inline bool is_crypto(KernelId k) { return k >= K_ETHASH; }
 

@@ -121,9 +121,11 @@ enum {
 /*
  * Create a plan for fusion `fusion_index` of `cfg`.
  *   preset    : "hfuse" | "hfuse_lb" | "vfuse" | "vfuse_lb" (main.cpp:182-193).
- *               Fused launches are built for the two hfuse presets; the vfuse
- *               presets only report their partition (launch returns
- *               HF_EUNSUPPORTED).
+ *               The hfuse presets partition the block's threads between the two
+ *               kernels; the vfuse presets are the reference's baseline in which
+ *               the same threads run kernel 1 and then kernel 2 (block =
+ *               max(d1, d2)).  The _lb variants differ only in the reported
+ *               launch_blocks hint.
  *   split_idx : the reference's enumeration index n (Split = 128*(n+1) threads
  *               for kernel 1, main.cpp:216-227); HF_SPLIT_TABLE keeps the
  *               YAML's BlockDim as the split; HF_SPLIT_EXECTIME re-splits in

@@ -136,7 +136,7 @@ def test_fused_sha256d_sia(cuda, cfg):
     want1 = oracle_hits(O.sha256d_search(h1, 5, 1 << 20, EASY16))
     want2 = oracle_hits(O.sia_search(h2, 9, (1 << 20) + 333, EASY16))
     i = cfg.find_fusion("sha256d_gpu_hash_shared", "sia_blake2b_gpu_hash")
-    for plan in (cfg.plan(i), cfg.plan(i, "hfuse", -1, 64), cfg.plan(i, "hfuse_lb", 0)):
+    for plan in (cfg.plan(i), cfg.plan(i, "hfuse", -1, 64), cfg.plan(i, "hfuse_lb", 0), cfg.plan(i, "vfuse")):
         r1, a1 = _search_pair_args(cuda, "sha256d_gpu_hash_shared", 1 << 20, 5)
         r2, a2 = _search_pair_args(cuda, "sia_blake2b_gpu_hash", (1 << 20) + 333, 9)
         plan.launch(a1, a2)

@@ -348,6 +348,31 @@ def test_fused_block_shapes(cuda, cfg, block):
         b.check()
 
 
+@pytest.mark.parametrize("preset", ["vfuse", "vfuse_lb"])
+def test_vertical_baseline_presets(cuda, cfg, preset):
+    """The reference's baseline: the same threads run kernel 1, then kernel 2 (block = max(d1, d2))."""
+    cases = [
+        ("im2col_kernel", "MaxPoolForward",
+         lambda: Im2col(cuda, 4, 16, 56, 56), lambda: MaxPool(cuda, 4, 16, 112, 112, (3, 3), (2, 2), (1, 1))),
+        ("batch_norm_collect_statistics_kernel", "upsample_nearest2d_out_frame",
+         lambda: BnStats(cuda, 16, 24, 28, 28), lambda: Upsample(cuda, 4, 16, 56, 56, (112, 112))),
+        ("kernelHistogram1D", "MaxPoolForward",
+         lambda: Histc(cuda, 1 << 21), lambda: MaxPool(cuda, 4, 32, 64, 64, (2, 2), (2, 2), (0, 0))),
+        ("kernelHistogram1D", "batch_norm_collect_statistics_kernel",
+         lambda: Histc(cuda, 1 << 20), lambda: BnStats(cuda, 8, 64, 14, 14)),
+    ]
+    for k1, k2, m1, m2 in cases:
+        plan = cfg.plan(cfg.find_fusion(k1, k2), preset)
+        part = plan.partition
+        assert list(part.lo) == [0, 0] and part.launch_threads == max(part.hi)
+        for grid in (0, 5):
+            a, b = m1(), m2()
+            plan.launch(a.args, b.args, grid_blocks=grid)
+            sync()
+            a.check()
+            b.check()
+
+
 def test_fused_barrier_modes(cuda, cfg):
     """hist + bn both synchronise: subset counters, the shared hardware barrier and the
     blockIdx fallback must all give the same results."""
