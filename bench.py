@@ -50,6 +50,8 @@ def parse():
                          "(default: the tuned split of the shipped fusion list)")
     ap.add_argument("--fused-only", action="store_true", help="launch only the fused kernel (profiling runs)")
     ap.add_argument("--search-log2", type=int, default=None, help="override log2 of the nonce ranges (debug)")
+    ap.add_argument("--extra-pairs", action="store_true",
+                    help="also time the other tensor pairs of the shipped fusion list (the reference's ml_fusion.yaml)")
     ap.add_argument("--calibrate-copy", type=int, default=0, metavar="MIB",
                     help="also run the plain copy kernel on MIB mebibytes (the unit HBM counters are scaled by)")
     return ap.parse_args()
@@ -86,48 +88,78 @@ def randn(shape, seed, mean, std, dev="cuda"):
     return torch.randn(shape, generator=g, device=dev, dtype=torch.float32) * std + mean
 
 
-def build_tensor_pairs(names):
+def kernel_workload(kname, variant=""):
+    """-> (make(i) -> dict(keep, args, read_bytes), algorithmic bytes) for one tensor kernel at its benchmark shape."""
     import torch
     from hfuse_amd import launcher as H
-    pairs = {}
 
     def nbytes(*ts):
         return sum(t.numel() * t.element_size() for t in ts)
 
-    if "im2col_maxpool" in names:
+    if kname == "im2col_kernel":
         def mk(i):
             x = rand((32, 64, 56, 56), SEED + 10 * i)
             col = torch.empty((32, 576, 3136), device="cuda")
+            return dict(keep=(x, col), read_bytes=nbytes(x), args=H.im2col_args(x, col))
+        return mk, 256901120
+    if kname == "MaxPoolForward" and variant == "k2":   # benchmark config 3
+        def mk(i):
+            y = rand((16, 128, 64, 64), SEED + 10 * i + 5)
+            val = torch.empty((16, 128, 32, 32), device="cuda")
+            idx = torch.empty((16, 128, 32, 32), dtype=torch.int64, device="cuda")
+            return dict(keep=(y, val, idx), read_bytes=nbytes(y),
+                        args=H.maxpool_args(y, val, idx, (2, 2), (2, 2), (0, 0)))
+        return mk, 58720256
+    if kname == "MaxPoolForward":                        # benchmark config 1
+        def mk(i):
             y = rand((32, 64, 112, 112), SEED + 10 * i + 1)
             val = torch.empty((32, 64, 56, 56), device="cuda")
             idx = torch.empty((32, 64, 56, 56), dtype=torch.int64, device="cuda")
-            return dict(keep=(x, col, y, val, idx), min_read=min(nbytes(x), nbytes(y)),
-                        a1=H.im2col_args(x, col), a2=H.maxpool_args(y, val, idx, (3, 3), (2, 2), (1, 1)))
-        pairs["im2col_maxpool"] = TensorPair("im2col_maxpool", "im2col_kernel", "MaxPoolForward", mk,
-                                             256901120, 179830784)
-    if "bn_upsample" in names:
+            return dict(keep=(y, val, idx), read_bytes=nbytes(y),
+                        args=H.maxpool_args(y, val, idx, (3, 3), (2, 2), (1, 1)))
+        return mk, 179830784
+    if kname == "batch_norm_collect_statistics_kernel":
         def mk(i):
             x = randn((32, 256, 28, 28), SEED + 10 * i + 2, 0.5, 2.0)
             mean = torch.empty(256, device="cuda")
             inv = torch.empty(256, device="cuda")
+            return dict(keep=(x, mean, inv), read_bytes=nbytes(x), args=H.bn_stats_args(x, mean, inv, 1e-5, 0.0))
+        return mk, 25692160
+    if kname == "upsample_nearest2d_out_frame":
+        def mk(i):
             u = rand((32, 64, 56, 56), SEED + 10 * i + 3)
             out = torch.empty((32, 64, 112, 112), device="cuda")
-            return dict(keep=(x, mean, inv, u, out), min_read=min(nbytes(x), nbytes(u)),
-                        a1=H.bn_stats_args(x, mean, inv, 1e-5, 0.0), a2=H.upsample_nearest_args(u, out))
-        pairs["bn_upsample"] = TensorPair("bn_upsample", "batch_norm_collect_statistics_kernel",
-                                          "upsample_nearest2d_out_frame", mk, 25692160, 128450560)
-    if "histc_maxpool" in names:
+            return dict(keep=(u, out), read_bytes=nbytes(u), args=H.upsample_nearest_args(u, out))
+        return mk, 128450560
+    if kname == "kernelHistogram1D":
         def mk(i):
             x = rand((1 << 26,), SEED + 10 * i + 4, 0.0, 1.0)
             hist = torch.zeros(1024, device="cuda")
-            y = rand((16, 128, 64, 64), SEED + 10 * i + 5)
-            val = torch.empty((16, 128, 32, 32), device="cuda")
-            idx = torch.empty((16, 128, 32, 32), dtype=torch.int64, device="cuda")
-            return dict(keep=(x, hist, y, val, idx), min_read=min(nbytes(x), nbytes(y)),
-                        a1=H.histc_args(x, hist, 1024, 0.0, 1.0), a2=H.maxpool_args(y, val, idx, (2, 2), (2, 2), (0, 0)))
-        pairs["histc_maxpool"] = TensorPair("histc_maxpool", "kernelHistogram1D", "MaxPoolForward", mk,
-                                            268439552, 58720256)
-    return pairs
+            return dict(keep=(x, hist), read_bytes=nbytes(x), args=H.histc_args(x, hist, 1024, 0.0, 1.0))
+        return mk, 268439552
+    raise KeyError(kname)
+
+
+def build_pair(name, k1, k2, v1="", v2=""):
+    mk1, b1 = kernel_workload(k1, v1)
+    mk2, b2 = kernel_workload(k2, v2)
+
+    def mk(i):
+        s1, s2 = mk1(i), mk2(i)
+        return dict(keep=(s1["keep"], s2["keep"]), min_read=min(s1["read_bytes"], s2["read_bytes"]),
+                    a1=s1["args"], a2=s2["args"])
+    return TensorPair(name, k1, k2, mk, b1, b2)
+
+
+BENCH_TENSOR_PAIRS = {
+    "im2col_maxpool": ("im2col_kernel", "MaxPoolForward", "", ""),
+    "bn_upsample": ("batch_norm_collect_statistics_kernel", "upsample_nearest2d_out_frame", "", ""),
+    "histc_maxpool": ("kernelHistogram1D", "MaxPoolForward", "", "k2"),
+}
+
+
+def build_tensor_pairs(names):
+    return {n: build_pair(n, *BENCH_TENSOR_PAIRS[n]) for n in names if n in BENCH_TENSOR_PAIRS}
 
 
 def candidate_plans(cfg, k1, k2, sweep):
@@ -421,6 +453,22 @@ def main():
         report[name] = r
         torch.cuda.empty_cache()
 
+    extra = {}
+    if args.extra_pairs:
+        tensor_kernels = {"im2col_kernel", "MaxPoolForward", "batch_norm_collect_statistics_kernel",
+                          "upsample_nearest2d_out_frame", "kernelHistogram1D"}
+        done = {(v[0], v[1]) for v in BENCH_TENSOR_PAIRS.values()}
+        for _, k1, k2 in cfg.fusions():
+            if k1 in tensor_kernels and k2 in tensor_kernels and (k1, k2) not in done:
+                pair = build_pair(f"{k1}+{k2}", k1, k2)
+                r = time_tensor_pair(cfg, pair, args.steps, args.warmup, sweep, False)
+                r.pop("plan")
+                r["fused_gbps"] = (pair.bytes1 + pair.bytes2) / (r["t_fused_ms"] * 1e-3) / 1e9
+                r["speedup_pct"] = (r["t_b2b_ms"] / r["t_fused_ms"] - 1.0) * 100.0
+                extra[pair.name] = r
+                del pair
+                torch.cuda.empty_cache()
+
     cpu = None
     if not args.no_cpu:
         from oracle import oracle as O
@@ -467,6 +515,8 @@ def main():
         "cpu_baseline": cpu,
         "pairs": report,
     }
+    if extra:
+        line["extra_pairs"] = extra
     print(json.dumps(line))
 
 
