@@ -131,6 +131,12 @@ def kernel_workload(kname, variant=""):
             out = torch.empty((32, 64, 112, 112), device="cuda")
             return dict(keep=(u, out), read_bytes=nbytes(u), args=H.upsample_nearest_args(u, out))
         return mk, 128450560
+    if kname == "upsample_bilinear2d_out_frame":
+        def mk(i):
+            u = rand((32, 64, 56, 56), SEED + 10 * i + 6)
+            out = torch.empty((32, 64, 112, 112), device="cuda")
+            return dict(keep=(u, out), read_bytes=nbytes(u), args=H.upsample_bilinear_args(u, out, False))
+        return mk, 128450560
     if kname == "kernelHistogram1D":
         def mk(i):
             x = rand((1 << 26,), SEED + 10 * i + 4, 0.0, 1.0)
@@ -456,7 +462,7 @@ def main():
     extra = {}
     if args.extra_pairs:
         tensor_kernels = {"im2col_kernel", "MaxPoolForward", "batch_norm_collect_statistics_kernel",
-                          "upsample_nearest2d_out_frame", "kernelHistogram1D"}
+                          "upsample_nearest2d_out_frame", "upsample_bilinear2d_out_frame", "kernelHistogram1D"}
         done = {(v[0], v[1]) for v in BENCH_TENSOR_PAIRS.values()}
         for _, k1, k2 in cfg.fusions():
             if k1 in tensor_kernels and k2 in tensor_kernels and (k1, k2) not in done:

@@ -78,6 +78,15 @@ class UpsampleNearestArgs(C.Structure):
                 ("width2", C.c_size_t), ("height_scale", C.c_float), ("width_scale", C.c_float)]
 
 
+class Accessor4(C.Structure):
+    _fields_ = [("data", C.c_void_p), ("sizes", C.c_int64 * 4), ("strides", C.c_int64 * 4)]
+
+
+class UpsampleBilinearArgs(C.Structure):
+    _fields_ = [("n", C.c_int), ("rheight", C.c_float), ("rwidth", C.c_float), ("align_corners", C.c_int),
+                ("idata", Accessor4), ("odata", Accessor4)]
+
+
 class TensorInfo(C.Structure):
     _fields_ = [("data", C.c_void_p), ("sizes", C.c_int64 * HF_MAX_TENSORINFO_DIMS),
                 ("strides", C.c_int64 * HF_MAX_TENSORINFO_DIMS), ("dims", C.c_int)]

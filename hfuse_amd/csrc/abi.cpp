@@ -42,6 +42,7 @@ const KernelName kNames[] = {
     {"MaxPoolForward", K_MAXPOOL},
     {"batch_norm_collect_statistics_kernel", K_BNSTATS},
     {"upsample_nearest2d_out_frame", K_UPSAMPLE_NEAREST},
+    {"upsample_bilinear2d_out_frame", K_UPSAMPLE_BILINEAR},
     {"kernelHistogram1D", K_HISTC},
     {"ethash_search", K_ETHASH},
     // the reference clones ethash_search so each pair has its own symbol (configs/ethash_sha256.yaml:7)
@@ -153,6 +154,7 @@ struct Prepared {
 
 static_assert(sizeof(hf_im2col_args) <= 512 && sizeof(hf_maxpool_args) <= 512 && sizeof(hf_bn_stats_args) <= 512 &&
                   sizeof(hf_upsample_nearest_args) <= 512 && sizeof(hf_histc_args) <= 512 &&
+                  sizeof(hf_upsample_bilinear_args) <= 512 &&
                   sizeof(EthashDevArgs) <= 512 && sizeof(Sha256dDevArgs) <= 512 && sizeof(Blake2bDevArgs) <= 512,
               "argument blob too small");
 
@@ -242,6 +244,37 @@ int prepare_upsample(const hf_upsample_nearest_args &a, Prepared &p) {
   return HF_OK;
 }
 
+int prepare_bilinear(const hf_upsample_bilinear_args &a, Prepared &p) {
+  const char *who = "upsample_bilinear2d_out_frame: ";
+  if (!a.idata.data || !a.odata.data) return fail(HF_EINVAL, std::string(who) + "null data pointer");
+  for (int i = 0; i < 4; i++)
+    if (a.idata.sizes[i] <= 0 || a.odata.sizes[i] <= 0) return fail(HF_EINVAL, std::string(who) + "empty tensor");
+  if (a.idata.sizes[0] != a.odata.sizes[0] || a.idata.sizes[1] != a.odata.sizes[1])
+    return fail(HF_EINVAL, std::string(who) + "batch / channel counts of input and output differ");
+  if ((int64_t)a.n != a.odata.sizes[2] * a.odata.sizes[3])
+    return fail(HF_EINVAL, std::string(who) + "n is not height2 * width2");
+  if (!(a.rheight >= 0.0f) || !(a.rwidth >= 0.0f)) return fail(HF_EINVAL, std::string(who) + "negative scale");
+  const int64_t total = a.odata.sizes[0] * a.odata.sizes[1] * a.odata.sizes[2] * a.odata.sizes[3];
+  const int64_t in_total = a.idata.sizes[0] * a.idata.sizes[1] * a.idata.sizes[2] * a.idata.sizes[3];
+  if (total >= (int64_t)1 << 32 || in_total >= (int64_t)1 << 32)
+    return fail(HF_EUNSUPPORTED, std::string(who) + "tensors of 2^32 elements or more are not built");
+  std::memcpy(p.blob, &a, sizeof a);
+  auto contiguous = [](const hf_accessor4 &t) {
+    return t.strides[3] == 1 && t.strides[2] == t.sizes[3] && t.strides[1] == t.sizes[2] * t.sizes[3] &&
+           t.strides[0] == t.sizes[1] * t.sizes[2] * t.sizes[3];
+  };
+  const bool fast = contiguous(a.idata) && contiguous(a.odata) && a.odata.sizes[3] % 4 == 0 && aligned16(a.odata.data) &&
+                    (a.idata.sizes[2] != a.odata.sizes[2] || a.idata.sizes[3] != a.odata.sizes[3] || aligned16(a.idata.data));
+  // exact 2x without align_corners: 0.5 * (dst + 0.5) - 0.5 is exact below 2^22 output columns / rows
+  const bool twice = fast && !a.align_corners && a.rheight == 0.5f && a.rwidth == 0.5f &&
+                     a.odata.sizes[2] == 2 * a.idata.sizes[2] && a.odata.sizes[3] == 2 * a.idata.sizes[3] &&
+                     a.idata.sizes[3] % 2 == 0 && ((uintptr_t)a.idata.data & 7) == 0 &&
+                     a.odata.sizes[2] < (1 << 22) && a.odata.sizes[3] < (1 << 22);
+  p.hint = twice ? HINT_BILINEAR_2X : fast ? HINT_BILINEAR_VEC4 : HINT_GENERIC;
+  p.items = twice ? (unsigned long long)total / 8 : fast ? (unsigned long long)total / 4 : (unsigned long long)total;
+  return HF_OK;
+}
+
 int prepare_histc(const hf_histc_args &a, Prepared &p) {
   if (!a.a.data || !a.b.data) return fail(HF_EINVAL, "kernelHistogram1D: null data pointer");
   if (a.nbins <= 0) return fail(HF_EINVAL, "kernelHistogram1D: bins must be > 0");
@@ -326,6 +359,7 @@ int prepare(KernelId id, const void *args, Prepared &p) {
     case K_BNSTATS: return prepare_bn(*static_cast<const hf_bn_stats_args *>(args), p);
     case K_UPSAMPLE_NEAREST: return prepare_upsample(*static_cast<const hf_upsample_nearest_args *>(args), p);
     case K_HISTC: return prepare_histc(*static_cast<const hf_histc_args *>(args), p);
+    case K_UPSAMPLE_BILINEAR: return prepare_bilinear(*static_cast<const hf_upsample_bilinear_args *>(args), p);
     case K_ETHASH: return prepare_ethash(*static_cast<const hf_ethash_args *>(args), p);
     case K_SHA256D: return prepare_sha256d(*static_cast<const hf_sha256d_args *>(args), p);
     case K_SIA_BLAKE2B: return prepare_blake2b(*static_cast<const hf_blake2b_args *>(args), true, p);
@@ -477,7 +511,7 @@ HF_API int hf_plan_create(const hf_config *cfg, int fusion_index, const char *pr
   for (int i = 0; i < 2; i++) {
     plan->rows[i] = *cfg->cfg.find(f.kernels[i]);
     if (!lookup_kernel(plan->rows[i].name, plan->ids[i])) {
-      int code = plan->rows[i].name == "upsample_bilinear2d_out_frame" ? HF_EUNSUPPORTED : HF_ENOTFOUND;
+      int code = HF_ENOTFOUND;
       std::string msg = "kernel '" + plan->rows[i].name + "' has no gfx950 implementation in this library";
       delete plan;
       return fail(code, msg);

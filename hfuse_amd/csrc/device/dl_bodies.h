@@ -13,7 +13,7 @@
 namespace hfuse {
 
 // Hints (0 always means the general path).
-enum { HINT_GENERIC = 0, HINT_IM2COL_3X3_S1P1 = 1, HINT_POOL_K3S2P1 = 1, HINT_POOL_K2S2P0 = 2, HINT_UP_2X = 1, HINT_BN_VEC4 = 1, HINT_HIST_VEC4 = 1, HINT_HIST_POW2 = 2 };
+enum { HINT_GENERIC = 0, HINT_IM2COL_3X3_S1P1 = 1, HINT_POOL_K3S2P1 = 1, HINT_POOL_K2S2P0 = 2, HINT_UP_2X = 1, HINT_BN_VEC4 = 1, HINT_HIST_VEC4 = 1, HINT_HIST_POW2 = 2, HINT_BILINEAR_VEC4 = 1, HINT_BILINEAR_2X = 2 };
 
 __device__ __forceinline__ f32x4 ld4(const float *p) { return *reinterpret_cast<const f32x4 *>(p); }
 
@@ -302,6 +302,195 @@ struct UpsampleNearestBody {
       const int y1 = min((int)floorf((float)y2 * a.height_scale), (int)a.height1 - 1);
       const int x1 = min((int)floorf((float)x2 * a.width_scale), (int)a.width1 - 1);
       a.odata[index] = a.idata[(c * a.height1 + y1) * a.width1 + x1];
+    }
+  }
+};
+
+// ----------------------------------------------------------------------------
+// upsample_bilinear2d_out_frame<float,float>  (argument list: scripts/data/ml-event.csv:9)
+//   src = align_corners ? scale*dst : max(scale*(dst+0.5)-0.5, 0); i1 = (int)src; l1 = src-i1
+//   out = h0*(w0*a + w1*b) + h1*(w0*c + w1*d)
+// Every product and sum is rounded on its own (rn_mul / rn_add below keep the compiler from
+// contracting them into FMAs), so results are the same bits as a plain fp32 CPU evaluation.
+// The original runs one thread per output pixel and loops over batch and channels; here the
+// flat range is all outputs, four neighbouring columns per work item where the output is
+// contiguous, which keeps the stores 16 bytes per lane and contiguous across the wave.
+// ----------------------------------------------------------------------------
+// Singly rounded fp32 operations: the pragma keeps the compiler from contracting a
+// product and the sum that uses it into one fused multiply-add (HIP's __fmul_rn and
+// __fadd_rn are plain operators, which the default -ffp-contract=fast may fuse).
+__device__ __forceinline__ float rn_mul(float x, float y) {
+#pragma clang fp contract(off)
+  return x * y;
+}
+__device__ __forceinline__ float rn_add(float x, float y) {
+#pragma clang fp contract(off)
+  return x + y;
+}
+__device__ __forceinline__ float rn_sub(float x, float y) {
+#pragma clang fp contract(off)
+  return x - y;
+}
+
+struct UpsampleBilinearBody {
+  using Args = hf_upsample_bilinear_args;
+  static constexpr bool kBarriers = false;
+  static constexpr bool kFlat = true;
+
+  static __device__ __forceinline__ float src_index(float scale, int dst, bool align) {
+    if (align) return rn_mul(scale, (float)dst);
+    const float s = rn_sub(rn_mul(scale, rn_add((float)dst, 0.5f)), 0.5f);
+    return s < 0.0f ? 0.0f : s;
+  }
+
+  static __device__ __forceinline__ float blend(float h0, float h1, float w0, float w1, float a, float b, float c,
+                                                float d) {
+    const float top = rn_add(rn_mul(w0, a), rn_mul(w1, b));
+    const float bot = rn_add(rn_mul(w0, c), rn_mul(w1, d));
+    return rn_add(rn_mul(h0, top), rn_mul(h1, bot));
+  }
+
+  // Exact 2x, align_corners off, contiguous NCHW, even input width.  A work item owns input
+  // row j, columns 2q and 2q+1 and writes output rows 2j and 2j+1, columns 4q..4q+3: those
+  // eight outputs read input rows j-1, j, j+1 (clamped) at columns 2q-1..2q+2.  Each row is
+  // one 8-byte load; the two outer columns are the neighbouring lanes' elements, moved with a
+  // wavefront-wide DPP shift (lanes 0 and 63 fetch theirs from memory).  Weights and source
+  // indices come from the same expressions as the general path, so the bits are the same.
+  // The trip count is wave-uniform so every lane's neighbour is live.
+  template <class SB>
+  static __device__ __forceinline__ void exact2x(const Args &a, SB &sb) {
+    const unsigned H1 = (unsigned)a.idata.sizes[2], W1 = (unsigned)a.idata.sizes[3];
+    const unsigned W2 = W1 * 2u;
+    const unsigned wq = W1 >> 1;
+    const unsigned NC = (unsigned)(a.idata.sizes[0] * a.idata.sizes[1]);
+    const unsigned n = NC * H1 * wq;
+    const unsigned stride = sb.gstride();
+    const unsigned lane = sb.lane();
+    for (unsigned first = sb.gtid() - lane; first < n; first += stride) {
+      const bool valid = first + lane < n;
+      const unsigned idx = valid ? first + lane : n - 1;
+      const unsigned q = idx % wq;
+      const unsigned t = idx / wq;
+      const unsigned j = t % H1;
+      const unsigned nc = t / H1;
+      const float *pl = a.idata.data + (size_t)nc * H1 * W1 + 2u * q;
+      const unsigned jr[3] = {j > 0 ? j - 1 : 0u, j, j + 1 < H1 ? j + 1 : j};
+      const bool has_left = q > 0, has_right = q + 1 < wq;
+      float wl[4], wr[4];  // weight of the left / right source column of output 4q+k
+#pragma unroll
+      for (int k = 0; k < 4; k++) {
+        const float w1r = src_index(a.rwidth, (int)(4u * q) + k, false);
+        wr[k] = rn_sub(w1r, (float)(int)w1r);
+        wl[k] = rn_sub(1.0f, wr[k]);
+      }
+      float hl[3][4];  // horizontally interpolated rows j-1, j, j+1
+#pragma unroll
+      for (int r = 0; r < 3; r++) {
+        const float *row = pl + (size_t)jr[r] * W1;
+        const float2 m = *reinterpret_cast<const float2 *>(row);
+        float left = dpp_f32<0x138>(m.y);   // wave_shr:1 -- lane-1's second column
+        float right = dpp_f32<0x130>(m.x);  // wave_shl:1 -- lane+1's first column
+        if (lane == 0 && has_left) left = row[-1];
+        if (lane == 63 && has_right) right = row[2];
+        // output 4q: source columns (2q-1, 2q), or (0, 1) with weights (1, 0) at the left edge
+        hl[r][0] = rn_add(rn_mul(wl[0], has_left ? left : m.x), rn_mul(wr[0], has_left ? m.x : m.y));
+        hl[r][1] = rn_add(rn_mul(wl[1], m.x), rn_mul(wr[1], m.y));
+        hl[r][2] = rn_add(rn_mul(wl[2], m.x), rn_mul(wr[2], m.y));
+        // output 4q+3: source columns (2q+1, 2q+2); the last column pairs with itself
+        hl[r][3] = rn_add(rn_mul(wl[3], m.y), rn_mul(wr[3], has_right ? right : m.y));
+      }
+      // output row 2j blends rows (j-1, j), or (0, 1) with weights (1, 0) at the top edge;
+      // output row 2j+1 blends rows (j, j+1), the last row with itself
+      const float s0 = src_index(a.rheight, (int)(2u * j), false), s1 = src_index(a.rheight, (int)(2u * j) + 1, false);
+      const float b0 = rn_sub(s0, (float)(int)s0), t0 = rn_sub(1.0f, b0);
+      const float b1 = rn_sub(s1, (float)(int)s1), t1 = rn_sub(1.0f, b1);
+      float o0[4], o1[4];
+#pragma unroll
+      for (int k = 0; k < 4; k++) {
+        o0[k] = rn_add(rn_mul(t0, hl[0][k]), rn_mul(b0, j > 0 ? hl[1][k] : hl[2][k]));
+        o1[k] = rn_add(rn_mul(t1, hl[1][k]), rn_mul(b1, hl[2][k]));
+      }
+      if (valid) {
+        float *out = a.odata.data + ((size_t)nc * (2u * H1) + 2u * j) * W2 + 4u * q;
+        st4(out, f32x4{o0[0], o0[1], o0[2], o0[3]});
+        st4(out + W2, f32x4{o1[0], o1[1], o1[2], o1[3]});
+      }
+    }
+  }
+
+  template <class SB>
+  static __device__ void run(const Args &a, SB &sb, unsigned char *, unsigned hint) {
+    const int H1 = (int)a.idata.sizes[2], W1 = (int)a.idata.sizes[3];
+    const int H2 = (int)a.odata.sizes[2], W2 = (int)a.odata.sizes[3];
+    const unsigned NC = (unsigned)(a.idata.sizes[0] * a.idata.sizes[1]);
+    const unsigned C = (unsigned)a.idata.sizes[1];
+    const bool align = a.align_corners != 0;
+    const bool same = H1 == H2 && W1 == W2;
+    if (hint == HINT_BILINEAR_2X) {
+      exact2x(a, sb);
+      return;
+    }
+    if (hint == HINT_BILINEAR_VEC4) {
+      // contiguous NCHW on both sides, W2 % 4 == 0, 16-byte aligned output
+      const unsigned wq = (unsigned)W2 >> 2;
+      const unsigned n4 = NC * (unsigned)H2 * wq;
+      const unsigned stride = sb.gstride();
+      for (unsigned idx = sb.gtid(); idx < n4; idx += stride) {
+        const unsigned xq = idx % wq;
+        const unsigned t = idx / wq;
+        const int y2 = (int)(t % (unsigned)H2);
+        const unsigned nc = t / (unsigned)H2;
+        const float *in = a.idata.data + (size_t)nc * H1 * W1;
+        f32x4 o;
+        if (same) {
+          o = ld4(in + (size_t)y2 * W1 + xq * 4);
+        } else {
+          const float h1r = src_index(a.rheight, y2, align);
+          const int y1 = (int)h1r;
+          const int y1p = (y1 < H1 - 1) ? 1 : 0;
+          const float h1l = rn_sub(h1r, (float)y1), h0l = rn_sub(1.0f, h1l);
+          const float *r0 = in + (size_t)y1 * W1, *r1 = r0 + (size_t)y1p * W1;
+          float v[4];
+#pragma unroll
+          for (int k = 0; k < 4; k++) {
+            const float w1r = src_index(a.rwidth, (int)(xq * 4) + k, align);
+            const int x1 = (int)w1r;
+            const int x1p = (x1 < W1 - 1) ? 1 : 0;
+            const float w1l = rn_sub(w1r, (float)x1), w0l = rn_sub(1.0f, w1l);
+            v[k] = blend(h0l, h1l, w0l, w1l, r0[x1], r0[x1 + x1p], r1[x1], r1[x1 + x1p]);
+          }
+          o = f32x4{v[0], v[1], v[2], v[3]};
+        }
+        st4(a.odata.data + (size_t)idx * 4, o);
+      }
+      return;
+    }
+    const unsigned total = NC * (unsigned)H2 * (unsigned)W2;
+    const unsigned stride = sb.gstride();
+    for (unsigned idx = sb.gtid(); idx < total; idx += stride) {
+      const int x2 = (int)(idx % (unsigned)W2);
+      const unsigned t = idx / (unsigned)W2;
+      const int y2 = (int)(t % (unsigned)H2);
+      const unsigned nc = t / (unsigned)H2;
+      const unsigned n = nc / C, c = nc - n * C;
+      const float *in = a.idata.data + (int64_t)n * a.idata.strides[0] + (int64_t)c * a.idata.strides[1];
+      float *out = a.odata.data + (int64_t)n * a.odata.strides[0] + (int64_t)c * a.odata.strides[1] +
+                   (int64_t)y2 * a.odata.strides[2] + (int64_t)x2 * a.odata.strides[3];
+      const int64_t sh = a.idata.strides[2], sw = a.idata.strides[3];
+      if (same) {
+        *out = in[y2 * sh + x2 * sw];
+        continue;
+      }
+      const float h1r = src_index(a.rheight, y2, align);
+      const int y1 = (int)h1r;
+      const int y1p = (y1 < H1 - 1) ? 1 : 0;
+      const float h1l = rn_sub(h1r, (float)y1), h0l = rn_sub(1.0f, h1l);
+      const float w1r = src_index(a.rwidth, x2, align);
+      const int x1 = (int)w1r;
+      const int x1p = (x1 < W1 - 1) ? 1 : 0;
+      const float w1l = rn_sub(w1r, (float)x1), w0l = rn_sub(1.0f, w1l);
+      *out = blend(h0l, h1l, w0l, w1l, in[y1 * sh + x1 * sw], in[y1 * sh + (x1 + x1p) * sw],
+                   in[(y1 + y1p) * sh + x1 * sw], in[(y1 + y1p) * sh + (x1 + x1p) * sw]);
     }
   }
 };

@@ -18,12 +18,13 @@ enum KernelId {
   K_SHA256D,
   K_SIA_BLAKE2B,
   K_BLAKE2B,
+  K_UPSAMPLE_BILINEAR,
   K_COUNT
 };
 
 enum FuseMode { MODE_HFUSE = 0, MODE_MATCHED = 1, MODE_BLOCKIDX = 2, MODE_VERTICAL = 3 };
 
-inline bool is_crypto(KernelId k) { return k >= K_ETHASH; }
+inline bool is_crypto(KernelId k) { return k >= K_ETHASH && k <= K_BLAKE2B; }
 
 // `dev_args` points at the device-side argument struct of kernel `k`
 // (hf_*_args for the tensor kernels, *DevArgs for the searches).

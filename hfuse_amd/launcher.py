@@ -210,6 +210,28 @@ def upsample_nearest_args(x, out, scales=None) -> L.UpsampleNearestArgs:
     return a
 
 
+def upsample_bilinear_args(x, out, align_corners=False, scales=None) -> L.UpsampleBilinearArgs:
+    """x [N,C,H1,W1], out [N,C,H2,W2] float32 (any strides); scales as PyTorch's area_pixel_compute_scale."""
+    import numpy as np
+    h1, w1 = x.shape[-2], x.shape[-1]
+    h2, w2 = out.shape[-2], out.shape[-1]
+    a = L.UpsampleBilinearArgs()
+    a.n = h2 * w2
+    if scales:
+        rh, rw = np.float32(scales[0]), np.float32(scales[1])
+    elif align_corners:
+        rh = np.float32(h1 - 1) / np.float32(h2 - 1) if h2 > 1 else np.float32(0)
+        rw = np.float32(w1 - 1) / np.float32(w2 - 1) if w2 > 1 else np.float32(0)
+    else:
+        rh, rw = np.float32(h1) / np.float32(h2), np.float32(w1) / np.float32(w2)
+    a.rheight, a.rwidth, a.align_corners = float(rh), float(rw), int(align_corners)
+    for acc, t in ((a.idata, x), (a.odata, out)):
+        acc.data = t.data_ptr()
+        acc.sizes[:] = list(t.shape)
+        acc.strides[:] = list(t.stride())
+    return a
+
+
 def histc_args(x, out, nbins, lo, hi) -> L.HistcArgs:
     a = L.HistcArgs()
     flat = x.reshape(-1)

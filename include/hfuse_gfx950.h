@@ -221,9 +221,9 @@ typedef struct {
 } hf_bn_stats_args;
 
 /*
- * upsample_nearest2d_out_frame<float> (PyTorch).  The reference fuses the
- * bilinear kernel (configs/ml_kernels.yaml:1-9); this build's contract asks for
- * nearest, whose argument list is the one below.
+ * upsample_nearest2d_out_frame<float> (PyTorch).  The reference's table lists
+ * the bilinear kernel (configs/ml_kernels.yaml:1-9, declared further down); the
+ * benchmarked pair uses nearest, whose argument list is the one below.
  */
 typedef struct {
   const float *idata;
@@ -231,6 +231,26 @@ typedef struct {
   size_t nc, height1, width1, height2, width2;
   float height_scale, width_scale;
 } hf_upsample_nearest_args;
+
+/* PackedTensorAccessor<float,4,DefaultPtrTraits,long> flattened. */
+typedef struct {
+  float *data;
+  int64_t sizes[4];
+  int64_t strides[4];
+} hf_accessor4;
+
+/*
+ * upsample_bilinear2d_out_frame<float,float> -- scripts/data/ml-event.csv:9,
+ * configs/ml_kernels.yaml:1-9.  n = height2 * width2 (the original runs one
+ * thread per output pixel and loops over batch and channels); rheight / rwidth
+ * are PyTorch's area_pixel_compute_scale values; align_corners is the bool.
+ */
+typedef struct {
+  int n;
+  float rheight, rwidth;
+  int align_corners;
+  hf_accessor4 idata, odata; /* [N, C, H, W] */
+} hf_upsample_bilinear_args;
 
 /* cuda::detail::TensorInfo<float,long> flattened. */
 #define HF_MAX_TENSORINFO_DIMS 8

@@ -262,6 +262,51 @@ ORC_API void orc_upsample_nearest2d(const float *idata, float *odata, size_t nc,
 }
 
 /*
+ * upsample_bilinear2d_out_frame<float,float> (PyTorch 1.4): signature
+ * scripts/data/ml-event.csv:9, table row configs/ml_kernels.yaml:1-9.
+ *   src = align_corners ? scale*dst : max(scale*(dst+0.5)-0.5, 0)
+ *   i1 = (int)src ; p = i1 < in-1 ; l1 = src - i1 ; l0 = 1 - l1
+ *   out = h0*(w0*a + w1*b) + h1*(w0*c + w1*d), every product and sum rounded to fp32
+ *   (no fused multiply-add), identical sizes copy through.
+ */
+static inline float bilinear_src(float scale, int dst, int align_corners) {
+  if (align_corners) return scale * (float)dst;
+  float s = scale * ((float)dst + 0.5f) - 0.5f;
+  return s < 0.0f ? 0.0f : s;
+}
+
+ORC_API void orc_upsample_bilinear2d(const float *idata, float *odata, int batch, int channels,
+                                     int h1, int w1, int h2, int w2, float rheight, float rwidth,
+                                     int align_corners) {
+#pragma omp parallel for schedule(static)
+  for (int64_t p = 0; p < (int64_t)batch * channels * h2; p++) {
+    int64_t nc = p / h2;
+    int y2 = (int)(p % h2);
+    const float *in = idata + nc * h1 * w1;
+    float *out = odata + (nc * h2 + y2) * (int64_t)w2;
+    if (h1 == h2 && w1 == w2) {
+      for (int x = 0; x < w2; x++) out[x] = in[(int64_t)y2 * w1 + x];
+      continue;
+    }
+    volatile float h1r = bilinear_src(rheight, y2, align_corners);
+    int y1 = (int)h1r;
+    int y1p = (y1 < h1 - 1) ? 1 : 0;
+    volatile float h1l = h1r - (float)y1, h0l = 1.0f - h1l;
+    for (int x2 = 0; x2 < w2; x2++) {
+      volatile float w1r = bilinear_src(rwidth, x2, align_corners);
+      int x1 = (int)w1r;
+      int x1p = (x1 < w1 - 1) ? 1 : 0;
+      volatile float w1l = w1r - (float)x1, w0l = 1.0f - w1l;
+      volatile float a = w0l * in[(int64_t)y1 * w1 + x1], b = w1l * in[(int64_t)y1 * w1 + x1 + x1p];
+      volatile float c = w0l * in[(int64_t)(y1 + y1p) * w1 + x1], d = w1l * in[(int64_t)(y1 + y1p) * w1 + x1 + x1p];
+      volatile float top = a + b, bot = c + d;
+      volatile float t0 = h0l * top, t1 = h1l * bot;
+      out[x2] = t0 + t1;
+    }
+  }
+}
+
+/*
  * kernelHistogram1D (PyTorch CUDA histc): call text scripts/configs/hist_norm.json:5.
  *   in range iff min <= v <= max ; bin = (int)((v-min)*nbins/(max-min)) in fp32,
  *   bin == nbins -> nbins-1 ; counts are fp32.

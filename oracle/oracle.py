@@ -151,6 +151,24 @@ def upsample_nearest2d(x, out_hw, scales=None):
     return out
 
 
+def upsample_bilinear2d(x, out_hw, align_corners=False, scales=None):
+    """x [N,C,H,W] float32 -> [N,C,H2,W2]; scales default to PyTorch's area_pixel_compute_scale."""
+    x, px = _f32(x)
+    n, c, h, w = x.shape
+    h2, w2 = out_hw
+    if scales:
+        rh, rw = np.float32(scales[0]), np.float32(scales[1])
+    elif align_corners:
+        rh = np.float32(h - 1) / np.float32(h2 - 1) if h2 > 1 else np.float32(0)
+        rw = np.float32(w - 1) / np.float32(w2 - 1) if w2 > 1 else np.float32(0)
+    else:
+        rh, rw = np.float32(h) / np.float32(h2), np.float32(w) / np.float32(w2)
+    out = np.empty((n, c, h2, w2), dtype=np.float32)
+    lib().orc_upsample_bilinear2d(px, out.ctypes.data_as(C.POINTER(C.c_float)), n, c, h, w, h2, w2,
+                                  C.c_float(rh), C.c_float(rw), int(align_corners))
+    return out
+
+
 def histc(x, nbins, lo, hi):
     x, px = _f32(np.ravel(x))
     out = np.zeros(nbins, dtype=np.float32)

@@ -9,7 +9,7 @@ import torch
 from hfuse_amd import _lib as L
 from hfuse_amd import launcher as H
 from oracle import oracle as O
-from util import normal, pool_out, rel_err, torch_bn_stats, torch_im2col, torch_maxpool, uniform
+from util import bilinear_tol, normal, pool_out, rel_err, torch_bn_stats, torch_im2col, torch_maxpool, uniform
 
 pytestmark = pytest.mark.gpu
 BN_TOL = 1e-5
@@ -65,6 +65,22 @@ class Upsample:
         want = torch.nn.functional.interpolate(self.x, size=self.out_hw, mode="nearest")
         assert torch.equal(self.out.cpu(), want), "upsample mismatch"
         assert np.array_equal(self.out.cpu().numpy(), O.upsample_nearest2d(self.x.numpy(), self.out_hw))
+        self.out.fill_(float("nan"))
+
+
+class Bilinear:
+    def __init__(self, dev, n, c, h, w, out_hw, align=False, seed=13):
+        self.x = uniform((n, c, h, w), seed)
+        self.out_hw, self.align = out_hw, align
+        self.xd = self.x.to(dev)
+        self.out = torch.full((n, c) + tuple(out_hw), float("nan"), device=dev)
+        self.args = H.upsample_bilinear_args(self.xd, self.out, align)
+
+    def check(self):
+        got = self.out.cpu().numpy()
+        assert np.array_equal(got, O.upsample_bilinear2d(self.x.numpy(), self.out_hw, self.align)), "bilinear mismatch"
+        want = torch.nn.functional.interpolate(self.x, size=self.out_hw, mode="bilinear", align_corners=self.align)
+        assert np.abs(got - want.numpy()).max() <= bilinear_tol(self.x.shape[2:], self.out_hw, self.align)
         self.out.fill_(float("nan"))
 
 
@@ -180,6 +196,67 @@ def test_upsample_nearest(cuda, shape, out):
     H.launch_native("upsample_nearest2d_out_frame", t.args)
     sync()
     t.check()
+
+
+@pytest.mark.parametrize("align", [False, True])
+@pytest.mark.parametrize("shape,out", [((8, 16, 56, 56), (112, 112)), ((2, 3, 5, 7), (10, 14)), ((1, 2, 4, 4), (7, 9)),
+                                       ((1, 1, 6, 5), (3, 4)), ((2, 2, 8, 12), (8, 12)), ((1, 2, 9, 9), (1, 1)),
+                                       # exact 2x with an even input width: the shifted-lane path, rows of 1, 3, 65
+                                       # and 100 work items so wavefront boundaries fall inside and between rows
+                                       ((1, 1, 1, 2), (2, 4)), ((2, 3, 5, 6), (10, 12)), ((3, 2, 7, 130), (14, 260)),
+                                       ((1, 5, 33, 200), (66, 400)), ((2, 2, 1, 64), (2, 128)),
+                                       ((1, 1, 6, 8), (12, 24)), ((1, 1, 6, 8), (18, 16))], ids=str)
+def test_upsample_bilinear(cuda, shape, out, align):
+    """Bit-exact against the oracle (no fused multiply-adds on either side), 2 ulp against PyTorch CPU."""
+    t = Bilinear(cuda, *shape, out, align)
+    H.launch_native("upsample_bilinear2d_out_frame", t.args)
+    sync()
+    t.check()
+
+
+def test_upsample_bilinear_signed_zeros(cuda):
+    """Bit patterns, not values: -0.0 inputs and the zero weights of the clamped edges."""
+    x = uniform((2, 2, 6, 8), 23)
+    x[x.abs() < 0.3] = 0.0
+    x[(x > 0.3) & (x < 0.5)] = -0.0
+    out = torch.empty((2, 2, 12, 16), device=cuda)
+    H.launch_native("upsample_bilinear2d_out_frame", H.upsample_bilinear_args(x.to(cuda), out, False))
+    sync()
+    want = O.upsample_bilinear2d(x.numpy(), (12, 16), False)
+    assert np.array_equal(out.cpu().numpy().view(np.uint32), want.view(np.uint32))
+
+
+def test_upsample_bilinear_strided_output(cuda):
+    x = uniform((2, 3, 6, 6), 17)
+    xd = x.to(cuda)
+    big = torch.zeros((2, 3, 12, 16), device=cuda)
+    view = big[:, :, :, 2:14]
+    H.launch_native("upsample_bilinear2d_out_frame", H.upsample_bilinear_args(xd, view, False))
+    sync()
+    assert np.array_equal(view.cpu().numpy(), O.upsample_bilinear2d(x.numpy(), (12, 12), False))
+    assert float(big[:, :, :, :2].abs().sum()) == 0.0 and float(big[:, :, :, 14:].abs().sum()) == 0.0
+
+
+def test_reference_ml_pairs_with_bilinear(cuda):
+    """The four pairs of the reference's ml_fusion.yaml that contain the bilinear kernel."""
+    from test_host_config import REFERENCE_ML_FUSION, REFERENCE_ML_KERNELS, REFERENCE_ML_PAIRS
+    ref_cfg = H.Config(REFERENCE_ML_FUSION, REFERENCE_ML_KERNELS)
+    made = []
+    makers = {
+        "im2col_kernel": lambda: Im2col(cuda, 2, 4, 12, 12),
+        "MaxPoolForward": lambda: MaxPool(cuda, 2, 4, 16, 16, (3, 3), (2, 2), (1, 1)),
+        "batch_norm_collect_statistics_kernel": lambda: BnStats(cuda, 4, 9, 6, 6),
+        "upsample_bilinear2d_out_frame": lambda: Bilinear(cuda, 4, 8, 28, 28, (56, 56) if len(made) % 2 else (42, 60)),
+        "kernelHistogram1D": lambda: Histc(cuda, 50000),
+    }
+    for i, (k1, k2) in enumerate(REFERENCE_ML_PAIRS):
+        for preset, idx in (("hfuse", L.HF_SPLIT_TABLE), ("hfuse", 0), ("vfuse", L.HF_SPLIT_TABLE)):
+            a, b = makers[k1](), makers[k2]()
+            made.append(i)
+            ref_cfg.plan(i, preset, idx).launch(a.args, b.args)
+            sync()
+            a.check()
+            b.check()
 
 
 @pytest.mark.parametrize("shape", [(32, 256, 28, 28), (4, 3, 5, 10), (2, 5, 7, 1), (3, 2, 3, 3), (64, 7, 4, 4)],

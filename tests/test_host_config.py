@@ -265,16 +265,8 @@ def test_barrier_policy(cfg):
     assert both.partition.barrier_mode == L.HF_BARRIER_MATCHED
 
 
-def test_unknown_and_unbuilt_kernels():
+def test_unknown_kernels_and_mixed_pairs():
     table = KERNELS_MAP + """
-upsample_bilinear2d_out_frame:
-  KernelName: upsample_bilinear2d_out_frame
-  HasBarriers: false
-  BlockDim:
-    X: 512
-    Y: 1
-    Z: 1
-  Reg: 43
 foo:
   KernelName: foo
   HasBarriers: false
@@ -283,16 +275,96 @@ foo:
     Y: 1
     Z: 1
   Reg: 8
+sia_blake2b_gpu_hash:
+  KernelName: sia_blake2b_gpu_hash
+  HasBarriers: false
+  BlockDim:
+    X: 128
+    Y: 1
+    Z: 1
+  Reg: 64
 """
-    fusion = ("- File: a\n  Kernels:\n    - MaxPoolForward\n    - upsample_bilinear2d_out_frame\n"
-              "- File: b\n  Kernels:\n    - foo\n    - MaxPoolForward\n")
+    fusion = ("- File: a\n  Kernels:\n    - foo\n    - MaxPoolForward\n"
+              "- File: b\n  Kernels:\n    - MaxPoolForward\n    - sia_blake2b_gpu_hash\n")
     cfg = Config(fusion, table)
     with pytest.raises(hfuse_amd.HfuseError) as e:
         cfg.plan(0)
-    assert e.value.code == L.HF_EUNSUPPORTED
+    assert e.value.code == L.HF_ENOTFOUND and "foo" in e.value.message
     with pytest.raises(hfuse_amd.HfuseError) as e:
         cfg.plan(1)
-    assert e.value.code == L.HF_ENOTFOUND
+    assert e.value.code == L.HF_EUNSUPPORTED
+
+
+# The reference's own two ML configuration files, restated in its schema (same kernel names,
+# block shapes, Reg and ExecTime as configs/ml_kernels.yaml; same ten pairs as configs/ml_fusion.yaml).
+REFERENCE_ML_KERNELS = """
+upsample_bilinear2d_out_frame:
+  KernelName: upsample_bilinear2d_out_frame
+  HasBarriers: false
+  BlockDim:
+    X: 512
+    Y: 1
+    Z: 1
+  Reg: 43
+  ExecTime: 77
+kernelHistogram1D:
+  KernelName: kernelHistogram1D
+  HasBarriers: false
+  BlockDim:
+    X: 512
+    Y: 1
+    Z: 1
+  Reg: 32
+  ExecTime: 1
+batch_norm_collect_statistics_kernel:
+  KernelName: batch_norm_collect_statistics_kernel
+  HasBarriers: false
+  BlockDim:
+    X: 32
+    Y: 16
+    Z: 1
+  Reg: 24
+  ExecTime: 52
+im2col_kernel:
+  KernelName: im2col_kernel
+  HasBarriers: false
+  BlockDim:
+    X: 512
+    Y: 1
+    Z: 1
+  Reg: 49
+  ExecTime: 31
+MaxPoolForward:
+  KernelName: MaxPoolForward
+  HasBarriers: false
+  BlockDim:
+    X: 256
+    Y: 1
+    Z: 1
+  Reg: 24
+  ExecTime: 95
+"""
+REFERENCE_ML_PAIRS = [
+    ("im2col_kernel", "MaxPoolForward"), ("im2col_kernel", "batch_norm_collect_statistics_kernel"),
+    ("im2col_kernel", "kernelHistogram1D"), ("im2col_kernel", "upsample_bilinear2d_out_frame"),
+    ("MaxPoolForward", "batch_norm_collect_statistics_kernel"), ("MaxPoolForward", "upsample_bilinear2d_out_frame"),
+    ("kernelHistogram1D", "MaxPoolForward"), ("kernelHistogram1D", "upsample_bilinear2d_out_frame"),
+    ("upsample_bilinear2d_out_frame", "batch_norm_collect_statistics_kernel"),
+    ("kernelHistogram1D", "batch_norm_collect_statistics_kernel"),
+]
+REFERENCE_ML_FUSION = "".join(f"- File: f{i}.cu\n  Kernels:\n   - {a}\n   - {b}\n" for i, (a, b) in enumerate(REFERENCE_ML_PAIRS))
+
+
+def test_reference_ml_configuration_plans_every_pair():
+    """All ten pairs of the reference's ML lists get a plan (bilinear upsampling included)."""
+    cfg = Config(REFERENCE_ML_FUSION, REFERENCE_ML_KERNELS)
+    assert cfg.num_fusions == 10
+    for i, (a, b) in enumerate(REFERENCE_ML_PAIRS):
+        part = cfg.plan(i).partition
+        assert part.name.decode() == f"{a}_{b}_fused_kernel_hfuse_table"
+        assert part.launch_threads in (768, 1024)
+        for idx in range(cfg.num_splits(i)):
+            assert cfg.plan(i, "hfuse_lb", idx).partition.hi[0] == 128 * (idx + 1)
 
 
 def test_launch_argument_errors_never_reach_the_gpu(cfg):

@@ -5,7 +5,7 @@ import pytest
 import torch
 
 from oracle import oracle as O
-from util import normal, pool_out, rel_err, torch_bn_stats, torch_im2col, torch_maxpool, uniform
+from util import bilinear_tol, normal, pool_out, rel_err, torch_bn_stats, torch_im2col, torch_maxpool, uniform
 
 IM2COL_CASES = [
     # (N, C, H, W, kernel, pad, stride, dil)
@@ -98,6 +98,38 @@ def test_upsample_2x_closed_form():
     got = O.upsample_nearest2d(x, (12, 16))
     hh, ww = np.meshgrid(np.arange(12) >> 1, np.arange(16) >> 1, indexing="ij")
     assert np.array_equal(got, x[:, :, hh, ww])
+
+
+BILINEAR_CASES = [((2, 3, 5, 7), (10, 14)), ((1, 2, 4, 4), (7, 9)), ((1, 1, 6, 5), (3, 4)), ((2, 2, 56, 56), (112, 112)),
+                  ((1, 1, 3, 3), (3, 3)), ((1, 1, 8, 8), (1, 1)), ((1, 2, 1, 5), (4, 5)), ((1, 3, 50, 50), (77, 131)),
+                  ((4, 8, 28, 28), (42, 60)), ((1, 1, 6, 8), (12, 24))]
+
+
+@pytest.mark.parametrize("align", [False, True])
+@pytest.mark.parametrize("shape,out", BILINEAR_CASES)
+def test_upsample_bilinear_vs_torch(shape, out, align):
+    """PyTorch CPU associates the four products differently and rounds the source index
+    differently, so agreement is to rounding (bound: util.bilinear_tol)."""
+    x = uniform(shape, 6)
+    got = O.upsample_bilinear2d(x.numpy(), out, align)
+    want = torch.nn.functional.interpolate(x, size=out, mode="bilinear", align_corners=align).numpy()
+    assert np.abs(got - want).max() <= bilinear_tol(shape[2:], out, align)
+
+
+def test_upsample_bilinear_closed_forms():
+    x = uniform((2, 3, 6, 8), 7).numpy()
+    assert np.array_equal(O.upsample_bilinear2d(x, (6, 8), False), x)            # same size: a copy
+    c = np.full((1, 2, 5, 7), 0.375, dtype=np.float32)
+    assert np.array_equal(O.upsample_bilinear2d(c, (11, 9), False), np.full((1, 2, 11, 9), 0.375, dtype=np.float32))
+    # align_corners on a 2 x 2 image: corners are kept, the centre of a 3 x 3 output is the mean
+    q = np.array([[[[0.0, 1.0], [2.0, 4.0]]]], dtype=np.float32)
+    o = O.upsample_bilinear2d(q, (3, 3), True)
+    assert o[0, 0, 0, 0] == 0.0 and o[0, 0, 0, 2] == 1.0 and o[0, 0, 2, 0] == 2.0 and o[0, 0, 2, 2] == 4.0
+    assert o[0, 0, 1, 1] == 1.75 and o[0, 0, 0, 1] == 0.5 and o[0, 0, 1, 0] == 1.0
+    # exact 2x without align_corners: interior weights are 0.25 / 0.75
+    r = np.arange(8, dtype=np.float32).reshape(1, 1, 1, 8)
+    o = O.upsample_bilinear2d(r, (1, 16), False)[0, 0, 0]
+    assert o[0] == 0.0 and o[1] == 0.25 and o[2] == 0.75 and o[3] == 1.25 and o[15] == 7.0
 
 
 @pytest.mark.parametrize("n,nbins,lo,hi", [(100000, 1024, 0.0, 1.0), (5000, 16, 0.0, 1.0), (70001, 256, -2.0, 2.0),

@@ -16,6 +16,7 @@ STRUCTS = {
     "MaxPoolForward": L.MaxPoolArgs,
     "batch_norm_collect_statistics_kernel": L.BnStatsArgs,
     "kernelHistogram1D": L.HistcArgs,
+    "upsample_bilinear2d_out_frame": L.UpsampleBilinearArgs,
     "ethash_search": L.EthashArgs,
     "sha256d_gpu_hash_shared": L.Sha256dArgs,
     "blake2b_gpu_hash": L.Blake2bArgs,

@@ -38,3 +38,17 @@ def rel_err(a, b):
     a = np.asarray(a, dtype=np.float64)
     b = np.asarray(b, dtype=np.float64)
     return float(np.max(np.abs(a - b) / np.maximum(np.abs(b), 1e-30)))
+
+
+def bilinear_tol(in_hw, out_hw, align):
+    """Bound on |oracle - PyTorch CPU| for bilinear upsampling of inputs in [-1, 1].
+
+    Both evaluate the same interpolant; they differ in how the four products are associated
+    (2 ulp of the value) and, when the size ratio is not a power of two, in the rounding of
+    the fp32 source index scale * (dst + 0.5) - 0.5, whose error of a few ulp of the index
+    (<= max(H1, W1)) is multiplied by the difference of two neighbouring pixels (<= 2)."""
+    def dyadic(i, o):
+        r = o / i
+        return r >= 1 and r == int(r) and int(r) & (int(r) - 1) == 0
+    exact = not align and dyadic(in_hw[0], out_hw[0]) and dyadic(in_hw[1], out_hw[1])
+    return 2.4e-7 if exact else 2.4e-7 * (1 + max(in_hw))
