@@ -29,7 +29,6 @@ VALU_PEAK_GOPS = 256 * 128 * 2.4  # 256 CUs x 128 lanes x 2.4 GHz int32 op/s in 
 # HBM bytes per launch of the headline fused kernel from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE, each
 # scaled by what the same counter reads for the plain copy kernel (profiles/bn_upsample_fused_hbm_traffic.md)
 HEADLINE_TRAFFIC_BYTES = {"bn_upsample": 156.83e6}
-SEED = 0x48467573
 
 # textbook primitive-op counts per hash (add / logic / rotate / shift = 1 each)
 OPS_SHA256D = 4336
@@ -57,115 +56,7 @@ def parse():
     return ap.parse_args()
 
 
-# ------------------------------------------------------------------ workloads
-class TensorPair:
-    """One tensor pair: `nsets` independent input/output sets so repeats miss the last-level cache."""
-
-    def __init__(self, name, k1, k2, make_set, bytes1, bytes2, min_read_footprint=600 << 20):
-        # Enough sets that even the smaller of the two read streams cycles through more bytes
-        # than the 256 MB memory-side cache holds, so neither kernel re-reads cached inputs.
-        self.name, self.k1, self.k2 = name, k1, k2
-        self.bytes1, self.bytes2 = bytes1, bytes2
-        self.sets = []
-        read_footprint = 0
-        while read_footprint < min_read_footprint or len(self.sets) < 2:
-            s = make_set(len(self.sets))
-            self.sets.append(s)
-            read_footprint += s["min_read"]
-        self.args1 = [s["a1"] for s in self.sets]
-        self.args2 = [s["a2"] for s in self.sets]
-
-
-def rand(shape, seed, lo=-1.0, hi=1.0, dev="cuda"):
-    import torch
-    g = torch.Generator(device=dev).manual_seed(seed)
-    return torch.rand(shape, generator=g, device=dev, dtype=torch.float32) * (hi - lo) + lo
-
-
-def randn(shape, seed, mean, std, dev="cuda"):
-    import torch
-    g = torch.Generator(device=dev).manual_seed(seed)
-    return torch.randn(shape, generator=g, device=dev, dtype=torch.float32) * std + mean
-
-
-def kernel_workload(kname, variant=""):
-    """-> (make(i) -> dict(keep, args, read_bytes), algorithmic bytes) for one tensor kernel at its benchmark shape."""
-    import torch
-    from hfuse_amd import launcher as H
-
-    def nbytes(*ts):
-        return sum(t.numel() * t.element_size() for t in ts)
-
-    if kname == "im2col_kernel":
-        def mk(i):
-            x = rand((32, 64, 56, 56), SEED + 10 * i)
-            col = torch.empty((32, 576, 3136), device="cuda")
-            return dict(keep=(x, col), read_bytes=nbytes(x), args=H.im2col_args(x, col))
-        return mk, 256901120
-    if kname == "MaxPoolForward" and variant == "k2":   # benchmark config 3
-        def mk(i):
-            y = rand((16, 128, 64, 64), SEED + 10 * i + 5)
-            val = torch.empty((16, 128, 32, 32), device="cuda")
-            idx = torch.empty((16, 128, 32, 32), dtype=torch.int64, device="cuda")
-            return dict(keep=(y, val, idx), read_bytes=nbytes(y),
-                        args=H.maxpool_args(y, val, idx, (2, 2), (2, 2), (0, 0)))
-        return mk, 58720256
-    if kname == "MaxPoolForward":                        # benchmark config 1
-        def mk(i):
-            y = rand((32, 64, 112, 112), SEED + 10 * i + 1)
-            val = torch.empty((32, 64, 56, 56), device="cuda")
-            idx = torch.empty((32, 64, 56, 56), dtype=torch.int64, device="cuda")
-            return dict(keep=(y, val, idx), read_bytes=nbytes(y),
-                        args=H.maxpool_args(y, val, idx, (3, 3), (2, 2), (1, 1)))
-        return mk, 179830784
-    if kname == "batch_norm_collect_statistics_kernel":
-        def mk(i):
-            x = randn((32, 256, 28, 28), SEED + 10 * i + 2, 0.5, 2.0)
-            mean = torch.empty(256, device="cuda")
-            inv = torch.empty(256, device="cuda")
-            return dict(keep=(x, mean, inv), read_bytes=nbytes(x), args=H.bn_stats_args(x, mean, inv, 1e-5, 0.0))
-        return mk, 25692160
-    if kname == "upsample_nearest2d_out_frame":
-        def mk(i):
-            u = rand((32, 64, 56, 56), SEED + 10 * i + 3)
-            out = torch.empty((32, 64, 112, 112), device="cuda")
-            return dict(keep=(u, out), read_bytes=nbytes(u), args=H.upsample_nearest_args(u, out))
-        return mk, 128450560
-    if kname == "upsample_bilinear2d_out_frame":
-        def mk(i):
-            u = rand((32, 64, 56, 56), SEED + 10 * i + 6)
-            out = torch.empty((32, 64, 112, 112), device="cuda")
-            return dict(keep=(u, out), read_bytes=nbytes(u), args=H.upsample_bilinear_args(u, out, False))
-        return mk, 128450560
-    if kname == "kernelHistogram1D":
-        def mk(i):
-            x = rand((1 << 26,), SEED + 10 * i + 4, 0.0, 1.0)
-            hist = torch.zeros(1024, device="cuda")
-            return dict(keep=(x, hist), read_bytes=nbytes(x), args=H.histc_args(x, hist, 1024, 0.0, 1.0))
-        return mk, 268439552
-    raise KeyError(kname)
-
-
-def build_pair(name, k1, k2, v1="", v2=""):
-    mk1, b1 = kernel_workload(k1, v1)
-    mk2, b2 = kernel_workload(k2, v2)
-
-    def mk(i):
-        s1, s2 = mk1(i), mk2(i)
-        return dict(keep=(s1["keep"], s2["keep"]), min_read=min(s1["read_bytes"], s2["read_bytes"]),
-                    a1=s1["args"], a2=s2["args"])
-    return TensorPair(name, k1, k2, mk, b1, b2)
-
-
-BENCH_TENSOR_PAIRS = {
-    "im2col_maxpool": ("im2col_kernel", "MaxPoolForward", "", ""),
-    "bn_upsample": ("batch_norm_collect_statistics_kernel", "upsample_nearest2d_out_frame", "", ""),
-    "histc_maxpool": ("kernelHistogram1D", "MaxPoolForward", "", "k2"),
-}
-
-
-def build_tensor_pairs(names):
-    return {n: build_pair(n, *BENCH_TENSOR_PAIRS[n]) for n in names if n in BENCH_TENSOR_PAIRS}
+from hfuse_amd.workloads import SEED, BENCH_TENSOR_PAIRS, TENSOR_KERNELS, build_pair, build_tensor_pairs  # noqa: E402
 
 
 def candidate_plans(cfg, k1, k2, sweep):
@@ -461,8 +352,7 @@ def main():
 
     extra = {}
     if args.extra_pairs:
-        tensor_kernels = {"im2col_kernel", "MaxPoolForward", "batch_norm_collect_statistics_kernel",
-                          "upsample_nearest2d_out_frame", "upsample_bilinear2d_out_frame", "kernelHistogram1D"}
+        tensor_kernels = set(TENSOR_KERNELS)
         done = {(v[0], v[1]) for v in BENCH_TENSOR_PAIRS.values()}
         for _, k1, k2 in cfg.fusions():
             if k1 in tensor_kernels and k2 in tensor_kernels and (k1, k2) not in done:

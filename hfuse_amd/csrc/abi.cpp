@@ -543,12 +543,20 @@ HF_API int hf_plan_create(const hf_config *cfg, int fusion_index, const char *pr
     delete plan;
     return fail(HF_EINVAL, "search kernels are built for fused blocks of at most 512 threads");
   }
+  if (f.lending >= 0) plan->lending = f.lending != 0;
   const bool b1 = body_has_barriers(plan->ids[0]), b2 = body_has_barriers(plan->ids[1]);
   // One barrier policy per pair: nothing to do when neither body synchronises;
   // an LDS-counter barrier scoped to the synchronising half otherwise.  (Both
   // tensor bodies that synchronise do so twice per block, so a pair of them may
   // also share the hardware barrier: HF_BARRIER_MATCHED via hf_plan_set_barrier_mode.)
   plan->barrier_mode = (b1 || b2) ? HF_BARRIER_SUBSET : HF_BARRIER_NONE;
+  if (f.barrier >= 0 && !p->base_line) {
+    rc = hf_plan_set_barrier_mode(plan, f.barrier);
+    if (rc != HF_OK) {
+      delete plan;
+      return rc;
+    }
+  }
   *out = plan;
   return HF_OK;
 }

@@ -154,8 +154,23 @@ bool parse_config(const char *fusion_yaml, const char *kernels_yaml, Config &cfg
           return false;
         }
       }
+      if (const YamlNode *ln = n.get("Lending")) {
+        if (ln->kind == YamlNode::Scalar && (ln->scalar == "true" || ln->scalar == "1")) f.lending = 1;
+        else if (ln->kind == YamlNode::Scalar && (ln->scalar == "false" || ln->scalar == "0")) f.lending = 0;
+        else { err = "fusion list: " + at(*ln) + "'Lending' must be true or false"; return false; }
+      }
+      if (const YamlNode *bn = n.get("Barrier")) {
+        static const char *const kModes[] = {"none", "matched", "subset", "blockidx"};  // HF_BARRIER_* order
+        for (int m = 0; m < 4; m++)
+          if (bn->kind == YamlNode::Scalar && bn->scalar == kModes[m]) f.barrier = m;
+        if (f.barrier < 0) {
+          err = "fusion list: " + at(*bn) + "'Barrier' must be one of none, matched, subset, blockidx";
+          return false;
+        }
+      }
       for (auto &kv : n.map)
-        if (kv.first != "File" && kv.first != "Kernels" && kv.first != "Split" && kv.first != "Threads") {
+        if (kv.first != "File" && kv.first != "Kernels" && kv.first != "Split" && kv.first != "Threads" &&
+            kv.first != "Lending" && kv.first != "Barrier") {
           err = "fusion list: " + at(kv.second) + "unknown key '" + kv.first + "'";
           return false;
         }

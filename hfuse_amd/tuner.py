@@ -1,0 +1,281 @@
+"""Split tuner: the reference's preset x split sweep as a launcher mode.
+
+The reference generates one fused kernel per split of the enumeration 128*(n+1) < d1+d2
+(tools/llvm-smart-fuser/main.cpp:215-236), builds and profiles each, and keeps the fastest.
+Here every split is a launch-time choice of the same compiled kernel, so the sweep is a loop of
+timed launches: block shapes (threads of kernel 1, threads of kernel 2) in wavefront multiples,
+wave lending on and off, and the barrier modes legal for the pair.  The winner is written back
+into the fusion list as the `Split:` / `Threads:` / `Lending:` / `Barrier:` keys the library applies when a
+plan is created with the table split.
+
+The register-cap half of the reference's experiments (its *_lb presets, `Reg` bound per
+kernel) has no launch-time counterpart: a gfx950 kernel's VGPR budget follows from its launch
+bound at compile time.  What a launch can still choose is how many blocks share a CU, which is
+the `grids` dimension of the sweep (blocks per CU for each half of the fused grid).
+
+    python -m hfuse_amd.tuner --out tuned_fusion.yaml            # all shipped tensor pairs
+    python -m hfuse_amd.tuner --only Im2ColMaxPool,SummaryMaxpool --out tuned.yaml
+"""
+from __future__ import annotations
+
+import argparse
+import os
+import re
+import statistics
+import sys
+from dataclasses import dataclass, field
+from typing import List, Optional, Sequence, Tuple
+
+from . import _lib as L
+from . import launcher as H
+
+WAVE = 64
+MAX_TENSOR_BLOCK = 1024
+MAX_SEARCH_BLOCK = 512
+
+
+@dataclass
+class Candidate:
+    threads1: int
+    threads2: int
+    lending: bool = True
+    barrier_mode: Optional[int] = None   # None: the library's choice for the pair
+    grids: Tuple[int, int] = (0, 0)      # (0, 0): the library's grids
+
+    def label(self) -> str:
+        s = f"{self.threads1}+{self.threads2}"
+        if not self.lending:
+            s += " nolend"
+        if self.barrier_mode is not None:
+            s += f" {BARRIER_NAMES[self.barrier_mode]}"
+        if self.grids != (0, 0):
+            s += f" grids{self.grids[0]}x{self.grids[1]}"
+        return s
+
+
+@dataclass
+class TuneResult:
+    file: str
+    kernels: Tuple[str, str]
+    best: Candidate
+    t_best_ms: float
+    t_table_ms: float                 # the untuned table split of the kernel table
+    t_b2b_ms: float                   # the two native launches back to back
+    table: List[Tuple[str, float]] = field(default_factory=list)   # (candidate label, ms) of the whole sweep
+
+    @property
+    def speedup_pct(self) -> float:
+        return (self.t_b2b_ms / self.t_best_ms - 1.0) * 100.0
+
+
+def block_candidates(cfg: H.Config, fusion_index: int, max_block: Optional[int] = None,
+                     step: int = WAVE) -> List[Tuple[int, int]]:
+    """Every (threads1, threads2) the pair can run with: positive multiples of `step` (itself a
+    multiple of the 64-lane wavefront) that divide by each kernel's BlockDim.Y, total <= max_block
+    (1024 for tensor pairs, 512 for the searches).  The reference's enumeration
+    (128, 256, ... of a fixed total) is the subset with threads1 + threads2 = d1 + d2."""
+    if step % WAVE:
+        raise ValueError("step must be a multiple of the 64-lane wavefront")
+    _, k1, k2 = cfg.fusion(fusion_index)
+    r1, r2 = cfg.kernel(k1), cfg.kernel(k2)
+    if max_block is None:
+        max_block = MAX_SEARCH_BLOCK if k1 in SEARCH_NAMES or k2 in SEARCH_NAMES else MAX_TENSOR_BLOCK
+    y1, y2 = r1.block_dim.y, r2.block_dim.y
+    out = []
+    for t1 in range(step, max_block, step):
+        if t1 % y1:
+            continue
+        for t2 in range(step, max_block - t1 + 1, step):
+            if t2 % y2 == 0:
+                out.append((t1, t2))
+    return out
+
+
+SEARCH_NAMES = {"ethash_search", "ethash_search2", "ethash_search3", "ethash_search4",
+                "sha256d_gpu_hash_shared", "sia_blake2b_gpu_hash", "blake2b_gpu_hash"}
+
+
+def _make_plan(cfg: H.Config, fusion_index: int, c: Candidate) -> H.Plan:
+    plan = cfg.plan(fusion_index, "hfuse", L.HF_SPLIT_TABLE)
+    plan.set_block(c.threads1, c.threads2)
+    plan.set_lending(c.lending)
+    if c.barrier_mode is not None:
+        plan.set_barrier_mode(c.barrier_mode)
+    if c.grids != (0, 0):
+        plan.set_grids(*c.grids)
+    return plan
+
+
+def tune(cfg: H.Config, fusion_index: int, args1: Sequence, args2: Sequence, *,
+         blocks: Optional[Sequence[Tuple[int, int]]] = None, lending: Sequence[bool] = (True, False),
+         barrier_modes: Sequence[Optional[int]] = (None,), grids: Sequence[Tuple[int, int]] = ((0, 0),),
+         probe_iters: int = 20, final_iters: int = 100, finalists: int = 4, warmup: int = 3,
+         grid_blocks: int = 0, verbose: bool = False) -> TuneResult:
+    """Sweep the candidates of one pair on the caller's argument sets and return the fastest.
+
+    args1[i] / args2[i] are argument structs of independent buffer sets the timed launches rotate
+    through (hf_time_pair).  Every candidate gets `probe_iters` launches; the `finalists` fastest
+    are timed again over `final_iters` launches in three interleaved rounds, together with the
+    back-to-back native launches and the untuned table split, and the median decides."""
+    file, k1, k2 = cfg.fusion(fusion_index)
+    if blocks is None:
+        blocks = block_candidates(cfg, fusion_index, step=2 * WAVE)
+    cands = [Candidate(t1, t2, ln, bm, g) for (t1, t2) in blocks for ln in lending for bm in barrier_modes
+             for g in grids]
+    probed = []
+    for c in cands:
+        try:
+            plan = _make_plan(cfg, fusion_index, c)
+        except H.HfuseError:
+            continue   # not legal for this pair (BlockDim.Y, barrier mode, block cap)
+        t = plan.time(3, args1, args2, warmup, probe_iters, grid_blocks) / probe_iters
+        probed.append((t, c, plan))
+        if verbose:
+            print(f"  {c.label():28s} {t * 1e3:9.2f} us", file=sys.stderr, flush=True)
+    if not probed:
+        raise RuntimeError(f"no legal candidate for {k1} + {k2}")
+    probed.sort(key=lambda r: r[0])
+    final = probed[:max(1, finalists)]
+    # Untuned reference point: the kernel table's own split, whatever the fusion entry says.
+    base_cfg_plan = cfg.plan(fusion_index, "hfuse", 0)
+    d1 = cfg.kernel(k1).block_dim
+    d2 = cfg.kernel(k2).block_dim
+    try:
+        base_cfg_plan.set_block(d1.x * d1.y * d1.z, d2.x * d2.y * d2.z)
+        base_ok = True
+    except H.HfuseError:
+        base_ok = False
+    samples = {i: [] for i in range(len(final))}
+    s_b2b, s_table = [], []
+    for _ in range(3):
+        for i, (_, _, plan) in enumerate(final):
+            samples[i].append(plan.time(3, args1, args2, 2, final_iters, grid_blocks) / final_iters)
+        s_b2b.append(final[0][2].time(2, args1, args2, 2, final_iters, grid_blocks) / final_iters)
+        if base_ok:
+            s_table.append(base_cfg_plan.time(3, args1, args2, 2, final_iters, grid_blocks) / final_iters)
+    med = sorted(((statistics.median(v), i) for i, v in samples.items()))
+    # Timings this close are the same speed: among them prefer the library's defaults
+    # (lending on, the pair's own barrier design) so that noise does not write keys.
+    near = [(t, i) for t, i in med if t <= med[0][0] * 1.005]
+    t_best, ibest = min(near, key=lambda r: ((not final[r[1]][1].lending) + (final[r[1]][1].barrier_mode is not None), r[0]))
+    return TuneResult(file=file, kernels=(k1, k2), best=final[ibest][1], t_best_ms=t_best,
+                      t_table_ms=statistics.median(s_table) if s_table else float("nan"),
+                      t_b2b_ms=statistics.median(s_b2b),
+                      table=[(c.label(), t) for t, c, _ in probed])
+
+
+# ------------------------------------------------------------------ fusion list rewriting
+_TUNED_KEY = re.compile(r"^\s+(Split|Threads|Lending|Barrier)\s*:")
+BARRIER_NAMES = {L.HF_BARRIER_NONE: "none", L.HF_BARRIER_MATCHED: "matched", L.HF_BARRIER_SUBSET: "subset",
+                 L.HF_BARRIER_BLOCKIDX: "blockidx"}
+
+
+def apply_to_fusion_yaml(text: str, tuned: dict) -> str:
+    """Return the fusion list `text` with the tuned keys of `tuned` {entry index: Candidate or None}
+    written into those entries; comments and every other line are kept.  None removes an entry's
+    tuned keys (the pair then runs at the kernel table's block shapes)."""
+    lines = text.splitlines()
+    starts = [i for i, ln in enumerate(lines) if ln.startswith("- ")]
+    out: List[str] = []
+    for n, s in enumerate(starts):
+        if n == 0:
+            out.extend(lines[:s])
+        e = starts[n + 1] if n + 1 < len(starts) else len(lines)
+        entry = lines[s:e]
+        if n in tuned:
+            entry = [ln for ln in entry if not _TUNED_KEY.match(ln)]
+            # keep trailing comments / blank lines (they belong to the next entry) after the new keys
+            tail = []
+            while entry and (not entry[-1].strip() or entry[-1].lstrip().startswith("#")):
+                tail.insert(0, entry.pop())
+            c = tuned[n]
+            if c is not None:
+                entry.append(f"  Split: {c.threads1}")
+                entry.append(f"  Threads: {c.threads1 + c.threads2}")
+                if not c.lending:
+                    entry.append("  Lending: false")
+                if c.barrier_mode is not None:
+                    entry.append(f"  Barrier: {BARRIER_NAMES[c.barrier_mode]}")
+            entry.extend(tail)
+        out.extend(entry)
+    if not starts:
+        out = lines
+    return "\n".join(out) + "\n"
+
+
+# ------------------------------------------------------------------ command line
+def _default_paths():
+    here = os.path.join(os.path.dirname(os.path.abspath(__file__)), "configs")
+    return os.path.join(here, "gfx950_fusion.yaml"), os.path.join(here, "gfx950_kernels.yaml")
+
+
+def main(argv=None) -> int:
+    fusion_default, kernels_default = _default_paths()
+    ap = argparse.ArgumentParser(description=__doc__.split("\n\n")[0])
+    ap.add_argument("--fusion", default=fusion_default, help="fusion list (YAML)")
+    ap.add_argument("--kernels", default=kernels_default, help="kernel table (YAML)")
+    ap.add_argument("--out", required=True, help="where to write the tuned fusion list")
+    ap.add_argument("--only", default="", help="comma list of File names or k1+k2 to tune (default: every tensor pair)")
+    ap.add_argument("--searches", action="store_true", help="also tune the nonce-search pairs (allocates a 4 GiB DAG)")
+    ap.add_argument("--search-log2", type=int, default=24, help="log2 of the nonce range of a search launch while tuning")
+    ap.add_argument("--step", type=int, default=128, help="granule of the block-shape sweep in threads")
+    ap.add_argument("--min-gain", type=float, default=1.0,
+                    help="keep an entry's current keys unless the winner beats the table split by this many percent")
+    ap.add_argument("--blockidx", action="store_true",
+                    help="also try the block-index partition (each workgroup runs one of the two kernels), "
+                         "written as 'Barrier: blockidx' where it wins")
+    ap.add_argument("--verbose", action="store_true")
+    args = ap.parse_args(argv)
+
+    import torch
+    from . import workloads as W
+    if not torch.cuda.is_available():
+        print("hfuse_amd.tuner: no GPU", file=sys.stderr)
+        return 2
+    text = open(args.fusion).read()
+    cfg = H.Config(text, open(args.kernels).read())
+    only = {s for s in args.only.split(",") if s}
+    tuned = {}
+    seen = set()
+    for i, (file, k1, k2) in enumerate(cfg.fusions()):
+        if only and file not in only and f"{k1}+{k2}" not in only:
+            continue
+        if (k1, k2) in seen:
+            continue
+        tensor = k1 in W.TENSOR_KERNELS and k2 in W.TENSOR_KERNELS
+        search = k1 in W.SEARCH_KERNELS and k2 in W.SEARCH_KERNELS
+        if not tensor and not (search and args.searches):
+            continue
+        seen.add((k1, k2))
+        print(f"[{i}] {file}: {k1} + {k2}", file=sys.stderr, flush=True)
+        blocks = block_candidates(cfg, i, step=args.step)
+        if tensor:
+            bench_variant = {v[:2]: v[2:] for v in W.BENCH_TENSOR_PAIRS.values()}.get((k1, k2), ("", ""))
+            pair = W.build_pair(file, k1, k2, *bench_variant)
+            r = tune(cfg, i, pair.args1, pair.args2, blocks=blocks,
+                     barrier_modes=(None, L.HF_BARRIER_BLOCKIDX) if args.blockidx else (None,), verbose=args.verbose)
+            del pair
+        else:
+            sp = W.SearchPair(k1, k2, args.search_log2, args.search_log2)
+            _, _, a1, a2 = sp.fresh()
+            r = tune(cfg, i, [a1], [a2], blocks=blocks, lending=(True,), probe_iters=1, final_iters=2,
+                     warmup=0, grid_blocks=sp.grid, verbose=args.verbose)
+            del sp
+        torch.cuda.empty_cache()
+        gain = (r.t_table_ms / r.t_best_ms - 1.0) * 100.0 if r.t_table_ms == r.t_table_ms else float("inf")
+        keep = gain >= args.min_gain
+        print(f"    best {r.best.label()}: {r.t_best_ms * 1e3:.2f} us, table split {r.t_table_ms * 1e3:.2f} us, "
+              f"back to back {r.t_b2b_ms * 1e3:.2f} us ({r.speedup_pct:+.1f} %)"
+              f"{'' if keep else ' -- within noise of the table split, keys left out'}", file=sys.stderr, flush=True)
+        # the same pair may be listed more than once (the reference's lists repeat pairs): tune once, write all
+        for j, (_, a, b) in enumerate(cfg.fusions()):
+            if (a, b) == (k1, k2):
+                tuned[j] = r.best if keep else None
+    with open(args.out, "w") as f:
+        f.write(apply_to_fusion_yaml(text, tuned))
+    print(f"wrote {args.out} ({len(tuned)} entries tuned)", file=sys.stderr)
+    return 0
+
+
+if __name__ == "__main__":
+    sys.exit(main())

@@ -75,10 +75,13 @@ typedef struct {
  * and a string-keyed map of kernel rows.  `kernels_yaml` may also be the older
  * per-pair form, a bare sequence of rows (configs/im2col_maxpool.yaml); then
  * `fusion_yaml` may be NULL and the single fusion is that list in order.
- * Two keys beyond the reference's schema are accepted in a fusion entry:
- * `Split: <threads>`, a tuned default for kernel 1's share of the block, and
- * `Threads: <threads>`, a tuned size of the whole fused block (kernel 2 gets
- * Threads - Split); both apply when a plan is created with HF_SPLIT_TABLE.
+ * Four keys beyond the reference's schema are accepted in a fusion entry
+ * (the split tuner writes them): `Split: <threads>`, a tuned default for
+ * kernel 1's share of the block, and `Threads: <threads>`, a tuned size of the
+ * whole fused block (kernel 2 gets Threads - Split); both apply when a plan is
+ * created with HF_SPLIT_TABLE.  `Lending: true|false` sets the plan's default
+ * for hf_plan_set_lending and `Barrier: none|matched|subset|blockidx` the one
+ * for hf_plan_set_barrier_mode (an illegal mode fails hf_plan_create).
  */
 HF_API int hf_config_load_text(const char *fusion_yaml, const char *kernels_yaml, hf_config **out);
 HF_API int hf_config_load_files(const char *fusion_path, const char *kernels_path, hf_config **out);
