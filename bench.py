@@ -102,6 +102,9 @@ def time_tensor_pair(cfg, pair, steps, warmup, sweep, fused_only, rounds=5):
         vplan = cfg.plan(cfg.find_fusion(pair.k1, pair.k2), "vfuse")
         res["t_vfuse_ms"] = statistics.median(
             [vplan.time(3, pair.args1, pair.args2, 2, per) / per for _ in range(3)])
+        # the two natives on two streams at once, the launch pattern of the reference's own traces
+        res["t_two_streams_ms"] = statistics.median(
+            [plan.time(4, pair.args1, pair.args2, 2, per) / per for _ in range(3)])
     res["split"] = label
     part = plan.partition
     res["fused_name"] = part.name.decode()
@@ -172,6 +175,7 @@ def run_search_pair(cfg, name, log2_a, log2_b, sweep, fused_only, iters=2):
     res["t_fused_ms"] = plan.time(3, [a1], [a2], 0, iters, grid) / iters
     if not fused_only:
         res["t_vfuse_ms"] = cfg.plan(cfg.find_fusion(k1, k2), "vfuse").time(3, [a1], [a2], 0, 1, grid)
+        res["t_two_streams_ms"] = base.time(4, [a1], [a2], 0, 1, grid)
     res["split"] = label
     part = plan.partition
     res["fused_name"] = part.name.decode()

@@ -793,8 +793,26 @@ HF_API int hf_launch_fused(const hf_plan *plan, const void *args1, const void *a
 HF_API int hf_time_pair(const hf_plan *plan, int mode, const void *const *args1, const void *const *args2, int nsets,
                         int warmup, int iters, int grid_blocks, void *stream_, float *elapsed_ms) {
   if (!plan || !args1 || !args2 || !elapsed_ms) return fail(HF_EINVAL, "null argument");
-  if (nsets <= 0 || iters <= 0 || warmup < 0 || mode < 0 || mode > 3) return fail(HF_EINVAL, "bad repetition arguments");
+  if (nsets <= 0 || iters <= 0 || warmup < 0 || mode < 0 || mode > 4) return fail(HF_EINVAL, "bad repetition arguments");
   hipStream_t stream = static_cast<hipStream_t>(stream_);
+  // mode 4: a second stream (default priority) and a fork / join event pair per repetition
+  hipStream_t side = nullptr;
+  hipEvent_t fork = nullptr, join = nullptr;
+  struct SideGuard {
+    hipStream_t &s;
+    hipEvent_t &a, &b;
+    ~SideGuard() {
+      if (a) (void)hipEventDestroy(a);
+      if (b) (void)hipEventDestroy(b);
+      if (s) (void)hipStreamDestroy(s);
+    }
+  } side_guard{side, fork, join};
+  if (mode == 4) {
+    hipError_t se = hipStreamCreateWithFlags(&side, hipStreamNonBlocking);
+    if (se == hipSuccess) se = hipEventCreateWithFlags(&fork, hipEventDisableTiming);
+    if (se == hipSuccess) se = hipEventCreateWithFlags(&join, hipEventDisableTiming);
+    if (se != hipSuccess) return hip_fail(se, "second stream");
+  }
   std::vector<Prepared> p1(nsets), p2(nsets);
   for (int i = 0; i < nsets; i++) {
     int rc = prepare(plan->ids[0], args1[i], p1[i]);
@@ -815,6 +833,18 @@ HF_API int hf_time_pair(const hf_plan *plan, int mode, const void *const *args1,
     if (mode == 1 || mode == 2) rc = do_launch_native(plan->ids[1], p2[s], g2, b2, stream);
     if (rc != HF_OK) return rc;
     if (mode == 3) rc = do_launch_fused(plan, p1[s], p2[s], grid_blocks, stream);
+    if (mode == 4) {
+      hipError_t se = hipEventRecord(fork, stream);
+      if (se == hipSuccess) se = hipStreamWaitEvent(side, fork, 0);
+      if (se != hipSuccess) return hip_fail(se, "fork");
+      rc = do_launch_native(plan->ids[0], p1[s], p1[s].exact_grid ? grid_blocks : 0, b1, stream);
+      if (rc != HF_OK) return rc;
+      rc = do_launch_native(plan->ids[1], p2[s], p2[s].exact_grid ? grid_blocks : 0, b2, side);
+      if (rc != HF_OK) return rc;
+      se = hipEventRecord(join, side);
+      if (se == hipSuccess) se = hipStreamWaitEvent(stream, join, 0);
+      if (se != hipSuccess) return hip_fail(se, "join");
+    }
     return rc;
   };
   for (int i = 0; i < warmup; i++) {

@@ -351,6 +351,9 @@ HF_API int hf_launch_fused(const hf_plan *plan, const void *args1, const void *a
  *   mode 0: native kernel 1      mode 1: native kernel 2
  *   mode 2: kernel 1 then kernel 2 back to back on `stream`
  *   mode 3: the fused kernel
+ *   mode 4: kernel 1 on `stream` and kernel 2 on a second stream of the
+ *           library's own, forked and joined with events every repetition
+ *           (the two-stream launch the reference's traces were taken with)
  * cycling through `nsets` argument sets (args1[i], args2[i]) so repeats do not
  * hit in the last-level cache, and returns the elapsed milliseconds measured
  * with HIP events recorded on `stream` around the timed launches.

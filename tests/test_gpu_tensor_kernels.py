@@ -491,3 +491,19 @@ def test_every_shipped_tensor_pair(cuda, cfg):
             b.check()
             n += 1
     assert n == 11  # the ten pairs of the reference list plus bn+upsample in benchmark order
+
+
+def test_time_pair_modes_leave_correct_results(cuda, cfg):
+    """All five timing modes (natives, back to back, fused, two streams) run the real kernels."""
+    i = cfg.find_fusion("im2col_kernel", "MaxPoolForward")
+    plan = cfg.plan(i)
+    for mode in range(5):
+        a, b = Im2col(cuda, 2, 4, 12, 12), MaxPool(cuda, 2, 4, 16, 16, (3, 3), (2, 2), (1, 1))
+        assert plan.time(mode, [a.args], [b.args], 1, 3) > 0
+        sync()
+        if mode != 1:
+            a.check()
+        if mode != 0:
+            b.check()
+    with pytest.raises(H.HfuseError):
+        plan.time(5, [a.args], [b.args], 0, 1)
