@@ -186,7 +186,9 @@ def derived_metrics(c: Dict[str, float], cus: int = 256, xcds: int = 8) -> Dict[
 
     GRBM_GUI_ACTIVE comes back summed over the XCDs; per-XCD busy cycles are its share.
       valu_busy_pct   (issue_slot_utilization)   100 * SQ_ACTIVE_INST_VALU / CUs / busy
-      mem_wait_pct    (stall_memory_dependency)  100 * SQ_WAIT_INST_ANY / SQ_WAVE_CYCLES
+      mem_stalled_pct (stall_memory_dependency)  rocprofv3's own derived MemUnitStalled, when collected
+      wait_issue_pct  (no nvprof counterpart)    100 * SQ_WAIT_INST_ANY / SQ_WAVE_CYCLES: wave-cycles spent
+                      waiting for an earlier instruction of any kind, other waves' turns on the SIMD included
       occupancy_pct   (achieved_occupancy)       100 * 4 * SQ_WAVE_CYCLES / busy / CUs / 32 wave slots"""
     out: Dict[str, float] = {}
     busy = c.get("GRBM_GUI_ACTIVE", 0.0) / xcds
@@ -195,7 +197,9 @@ def derived_metrics(c: Dict[str, float], cus: int = 256, xcds: int = 8) -> Dict[
     if busy > 0 and "SQ_WAVE_CYCLES" in c:
         out["occupancy_pct"] = 400.0 * c["SQ_WAVE_CYCLES"] / busy / cus / 32
     if c.get("SQ_WAVE_CYCLES", 0.0) > 0 and "SQ_WAIT_INST_ANY" in c:
-        out["mem_wait_pct"] = 100.0 * c["SQ_WAIT_INST_ANY"] / c["SQ_WAVE_CYCLES"]
+        out["wait_issue_pct"] = 100.0 * c["SQ_WAIT_INST_ANY"] / c["SQ_WAVE_CYCLES"]
+    if "MemUnitStalled" in c:
+        out["mem_stalled_pct"] = c["MemUnitStalled"]
     if "SQ_WAVES" in c:
         out["waves"] = c["SQ_WAVES"]
     if "SQ_INSTS_VALU" in c:
@@ -246,7 +250,8 @@ def render_exec_table(table, fmt: str = "md") -> str:
     return "\n".join(lines)
 
 
-_METRIC_COLS = (("valu_busy_pct", "VALU busy %", "{:.1f}"), ("mem_wait_pct", "waiting %", "{:.1f}"),
+_METRIC_COLS = (("valu_busy_pct", "VALU busy %", "{:.1f}"), ("mem_stalled_pct", "mem unit stalled %", "{:.1f}"),
+                ("wait_issue_pct", "waiting on issue %", "{:.1f}"),
                 ("occupancy_pct", "occupancy %", "{:.1f}"), ("waves", "waves", "{:.0f}"),
                 ("valu_insts", "VALU insts", "{:.0f}"), ("fetch_kib", "FETCH_SIZE KiB", "{:.1f}"),
                 ("write_kib", "WRITE_SIZE KiB", "{:.1f}"))

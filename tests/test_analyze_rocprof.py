@@ -93,8 +93,8 @@ def test_metric_table(tmp_path):
     m = rows[0][2]
     # busy cycles per XCD = 8000 / 8 = 1000: 253440 / 256 CUs / 1000 = 99 %; 4 * 1474560 / 1000 / 256 / 32 = 72 %
     assert m["valu_busy_pct"] == pytest.approx(99.0) and m["occupancy_pct"] == pytest.approx(72.0)
-    assert m["mem_wait_pct"] == pytest.approx(10.0) and m["waves"] == 4096
-    assert rows[1][2]["valu_busy_pct"] == pytest.approx(50.0) and "mem_wait_pct" not in rows[1][2]
+    assert m["wait_issue_pct"] == pytest.approx(10.0) and m["waves"] == 4096
+    assert rows[1][2]["valu_busy_pct"] == pytest.approx(50.0) and "wait_issue_pct" not in rows[1][2]
     md = A.render_metric_table(rows)
     assert "| SHA256 | ST | 99.0 | 10.0 | 72.0 | 4096 |" in md and "| SHA256+Blake2B | HF@256 | 50.0 | * | 40.0 | 8192 |" in md
     assert A.agent_shape(str(p)) == (256, 8)   # no agent_info.csv beside it: MI355X
