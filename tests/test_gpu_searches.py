@@ -226,3 +226,21 @@ def test_every_shipped_search_pair(cuda, cfg):
             assert H.read_search_results(r2) == native[k2], (k1, k2)
             n += 1
     assert n == 7
+
+
+def test_zero_nonces_find_nothing(cuda, cfg):
+    hdr = O.seeded_bytes(80, SEED + 5)
+    H.sha256d_set_block(hdr, EASY12)
+    H.sia_blake2b_set_block(O.seeded_bytes(80, SEED + 6))
+    r1, r2 = H.new_search_results(), H.new_search_results()
+    H.launch_native("sha256d_gpu_hash_shared", H.sha256d_args(r1, 0, 0))
+    H.launch_native("sia_blake2b_gpu_hash", H.blake2b_args(r2, 0, 0, EASY12))
+    sync()
+    assert H.read_search_results(r1)[0] == 0 and H.read_search_results(r2)[0] == 0
+    # an empty half next to a working one: the working half's found set is unchanged
+    i = cfg.find_fusion("sha256d_gpu_hash_shared", "sia_blake2b_gpu_hash")
+    cfg.plan(i).launch(H.sha256d_args(r1, 1 << 14, 0), H.blake2b_args(r2, 0, 0, EASY12))
+    sync()
+    want = oracle_hits(O.sha256d_search(hdr, 0, 1 << 14, EASY12))
+    assert want[0] > 0 and H.read_search_results(r1) == want
+    assert H.read_search_results(r2)[0] == 0

@@ -507,3 +507,44 @@ def test_time_pair_modes_leave_correct_results(cuda, cfg):
             b.check()
     with pytest.raises(H.HfuseError):
         plan.time(5, [a.args], [b.args], 0, 1)
+
+
+def test_empty_work_is_a_no_op(cuda, cfg):
+    """Zero work items (im2col with n = 0, a histogram of nothing) return without touching their
+    outputs, alone and as one half of a fused launch; kernels whose PyTorch callers refuse empty
+    tensors (pooling, upsampling) refuse them here too."""
+    buf = torch.zeros(4096, device=cuda)
+    out = torch.full((4096,), 7.0, device=cuda)
+    a = H.im2col_args(buf[:64].reshape(1, 8, 8), out)
+    a.n = 0
+    H.launch_native("im2col_kernel", a)
+    h = H.histc_args(buf[:64], out[:16], 16, 0.0, 1.0)
+    h.total_elements = 0
+    h.b.sizes[0] = 0
+    H.launch_native("kernelHistogram1D", h)
+    sync()
+    assert float(out.min()) == 7.0 and float(out.max()) == 7.0
+    idx = torch.zeros(16, dtype=torch.int64, device=cuda)
+    m = H.maxpool_args(buf[:64].reshape(1, 1, 8, 8), out[:16].reshape(1, 1, 4, 4), idx.reshape(1, 1, 4, 4),
+                       (2, 2), (2, 2), (0, 0))
+    m.nthreads = 0
+    m.num = 0
+    u = H.upsample_nearest_args(buf[:64].reshape(1, 1, 8, 8), out[:256].reshape(1, 1, 16, 16))
+    u.nc = 0
+    for name, args in (("MaxPoolForward", m), ("upsample_nearest2d_out_frame", u)):
+        with pytest.raises(H.HfuseError) as e:
+            H.launch_native(name, args)
+        assert e.value.code == L.HF_EINVAL
+    # an empty half next to a working one, thread partition and block-index partition
+    i = cfg.find_fusion("im2col_kernel", "MaxPoolForward")
+    j = cfg.find_fusion("kernelHistogram1D", "MaxPoolForward")
+    for mode in (None, L.HF_BARRIER_BLOCKIDX):
+        for fusion, empty in ((i, a), (j, h)):
+            plan = cfg.plan(fusion)
+            if mode is not None:
+                plan.set_barrier_mode(mode)
+            pool = MaxPool(cuda, 2, 4, 16, 16, (2, 2), (2, 2), (0, 0))
+            plan.launch(empty, pool.args)
+            sync()
+            pool.check()
+    assert float(out.min()) == 7.0 and float(out.max()) == 7.0
