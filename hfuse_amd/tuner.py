@@ -218,7 +218,7 @@ def main(argv=None) -> int:
     ap.add_argument("--only", default="", help="comma list of File names or k1+k2 to tune (default: every tensor pair)")
     ap.add_argument("--searches", action="store_true", help="also tune the nonce-search pairs (allocates a 4 GiB DAG)")
     ap.add_argument("--search-log2", type=int, default=24, help="log2 of the nonce range of a search launch while tuning")
-    ap.add_argument("--step", type=int, default=128, help="granule of the block-shape sweep in threads")
+    ap.add_argument("--step", type=int, default=64, help="granule of the block-shape sweep in threads")
     ap.add_argument("--min-gain", type=float, default=1.0,
                     help="keep an entry's current keys unless the winner beats the table split by this many percent")
     ap.add_argument("--blockidx", action="store_true",
@@ -233,7 +233,11 @@ def main(argv=None) -> int:
         print("hfuse_amd.tuner: no GPU", file=sys.stderr)
         return 2
     text = open(args.fusion).read()
-    cfg = H.Config(text, open(args.kernels).read())
+    # Measure on the list without anybody's tuned keys, so that "the table split" and every
+    # candidate start from the library's defaults; the keys of entries that are not re-tuned
+    # are kept in the output, which is written from the original text.
+    entries = sum(1 for ln in text.splitlines() if ln.startswith("- "))
+    cfg = H.Config(apply_to_fusion_yaml(text, {n: None for n in range(entries)}), open(args.kernels).read())
     only = {s for s in args.only.split(",") if s}
     tuned = {}
     seen = set()

@@ -59,6 +59,18 @@ def test_apply_to_fusion_yaml_round_trip():
     assert T.apply_to_fusion_yaml(fusion, {}) == fusion if fusion.endswith("\n") else True
 
 
+def test_stripping_every_entry_gives_the_untuned_list():
+    fusion, kernels = shipped()
+    n = fusion.count("- File:")
+    clean = T.apply_to_fusion_yaml(fusion, {i: None for i in range(n)})
+    body = [ln for ln in clean.splitlines() if not ln.lstrip().startswith("#")]
+    assert not any(ln.split(":")[0].strip() in ("Split", "Threads", "Lending", "Barrier") for ln in body)
+    cfg = H.Config(clean, kernels)
+    assert cfg.fusions() == H.Config(fusion, kernels).fusions()
+    p = cfg.plan(cfg.find_fusion("kernelHistogram1D", "MaxPoolForward")).partition
+    assert (p.hi[0] - p.lo[0], p.hi[1] - p.lo[1]) == (512, 256)
+
+
 def test_barrier_key():
     _, kernels = shipped()
     base = "- File: a\n  Kernels:\n    - im2col_kernel\n    - MaxPoolForward\n"
