@@ -130,16 +130,17 @@ void host_sha256_compress(uint32_t st[8], const uint32_t blk[16]) {
 }
 
 // ------------------------------------------------------------ device facts
-int g_cu_count = 0;
+// Compute units of the current device, asked once (function-local static: thread-safe).
 int cu_count() {
-  if (g_cu_count == 0) {
+  static const int count = [] {
     int dev = 0;
     hipDeviceProp_t prop;
-    if (hipGetDevice(&dev) == hipSuccess && hipGetDeviceProperties(&prop, dev) == hipSuccess)
-      g_cu_count = prop.multiProcessorCount;
-    if (g_cu_count <= 0) g_cu_count = 256;
-  }
-  return g_cu_count;
+    if (hipGetDevice(&dev) == hipSuccess && hipGetDeviceProperties(&prop, dev) == hipSuccess &&
+        prop.multiProcessorCount > 0)
+      return prop.multiProcessorCount;
+    return 256;  // MI355X
+  }();
+  return count;
 }
 
 // ------------------------------------------------------- argument validation
@@ -399,6 +400,8 @@ int do_launch_native(KernelId id, const Prepared &p, int grid_blocks, unsigned b
   else if (p.exact_grid) grid = kDefaultEthashGrid;
   else grid = default_grid(p, block, block);
   if (!p.exact_grid && p.items == 0) return HF_OK;  // nothing to do
+  if ((unsigned long long)grid * block > 0xFFFFFFFFull)
+    return fail(HF_EINVAL, "grid_blocks * block threads must fit 32 bits (the bodies index work items with 32-bit counters)");
   hipError_t e = is_crypto(id) ? launch_native_crypto(id, p.blob, p.hint, grid, block, p.lds, stream)
                                : launch_native_dl(id, p.blob, p.hint, grid, block, p.lds, stream);
   if (e != hipSuccess) return hip_fail(e, "native launch");
@@ -722,6 +725,9 @@ int do_launch_fused(const hf_plan *plan, const Prepared &p1, const Prepared &p2,
   g.lend = 0;
   const bool crypto = is_crypto(plan->ids[0]);
   const unsigned exact = grid_blocks > 0 ? (unsigned)grid_blocks : kDefaultEthashGrid;
+  if ((unsigned long long)std::max(exact, std::max(plan->grid_override[0], plan->grid_override[1])) * (g.d1 + g.d2) >
+      0xFFFFFFFFull)
+    return fail(HF_EINVAL, "grid_blocks * block threads must fit 32 bits (the bodies index work items with 32-bit counters)");
   hipError_t e;
   if (plan->preset->base_line) {
     // Vertical baseline: both kernels start at thread 0 of a block of max(d1, d2) threads.

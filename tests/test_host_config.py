@@ -396,6 +396,16 @@ def test_launch_argument_errors_never_reach_the_gpu(cfg):
     assert b"max must be larger than min" in lib.hf_last_error()
     v = cfg.plan(0, "vfuse")
     assert lib.hf_launch_fused(v._h, C.byref(a), C.byref(b), 0, None) in (L.HF_EINVAL, L.HF_EUNSUPPORTED)
+    # a grid whose thread count does not fit the bodies' 32-bit work-item counters
+    a.height_col, a.width_col = 8, 8
+    assert lib.hf_launch_native(b"im2col_kernel", C.byref(a), 1 << 23, 1024, None) == L.HF_EINVAL
+    assert b"32 bits" in lib.hf_last_error()
+    b.bottom_data = b.top_data = b.top_mask = 256
+    b.nthreads, b.num, b.channels, b.height, b.width, b.pooled_height, b.pooled_width = 16, 1, 1, 8, 8, 4, 4
+    b.kernel_h = b.kernel_w = b.stride_h = b.stride_w = 2
+    b.dilation_h = b.dilation_w = 1
+    assert lib.hf_launch_fused(plan._h, C.byref(a), C.byref(b), 1 << 23, None) == L.HF_EINVAL
+    assert b"32 bits" in lib.hf_last_error()
 
 
 def test_header_symbols_are_all_exported():
