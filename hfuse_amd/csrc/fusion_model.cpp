@@ -57,6 +57,13 @@ bool parse_row(const YamlNode &n, bool reg_required, KernelRow &row, std::string
     err = at(n) + "missing or invalid required key 'BlockDim' {X, Y, Z}";
     return false;
   }
+  // A block of zero threads divides by zero further on; more than 1024 cannot be launched.
+  if (row.block_dim.x == 0 || row.block_dim.y == 0 || row.block_dim.z == 0 || row.block_dim.x > kMaxBlock ||
+      row.block_dim.y > kMaxBlock || row.block_dim.z > kMaxBlock ||
+      (uint64_t)row.block_dim.x * row.block_dim.y * row.block_dim.z > kMaxBlock) {
+    err = at(*bd) + "'BlockDim' must be 1..1024 threads in total, no component 0";
+    return false;
+  }
   const YamlNode *reg = n.get("Reg");
   if (reg) {
     if (!to_uint(reg, row.reg)) { err = at(n) + "invalid 'Reg'"; return false; }
