@@ -6,6 +6,7 @@
 #include <cmath>
 #include <cstring>
 #include <fstream>
+#include <initializer_list>
 #include <mutex>
 #include <sstream>
 #include <string>
@@ -161,24 +162,42 @@ static_assert(sizeof(hf_im2col_args) <= 512 && sizeof(hf_maxpool_args) <= 512 &&
 
 bool aligned16(const void *p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
 
+// Every extent, stride and geometry value a caller passes is bounded before it is multiplied:
+// one value below 2^31, products through checked multiplication, so no validator can overflow
+// or divide by a wrapped zero whatever the argument struct holds.
+constexpr int64_t kMaxExtent = (int64_t)1 << 31;
+constexpr int64_t kMaxOffset = (int64_t)1 << 46;  // elements; far beyond 288 GB of fp32
+bool extent_ok(int64_t v) { return v > 0 && v < kMaxExtent; }
+bool pad_ok(int64_t v) { return v >= 0 && v < kMaxExtent; }
+// out = product of the arguments, false on overflow of int64 or beyond kMaxOffset
+bool product(int64_t &out, std::initializer_list<int64_t> factors) {
+  out = 1;
+  for (int64_t f : factors)
+    if (f < 0 || __builtin_mul_overflow(out, f, &out) || out > kMaxOffset) return false;
+  return true;
+}
+
 int prepare_im2col(const hf_im2col_args &a, Prepared &p) {
   if (!a.data_im || !a.data_col) return fail(HF_EINVAL, "im2col_kernel: null data pointer");
-  if (a.n < 0 || a.height <= 0 || a.width <= 0 || a.kernel_h <= 0 || a.kernel_w <= 0 || a.stride_h <= 0 ||
-      a.stride_w <= 0 || a.dilation_h <= 0 || a.dilation_w <= 0 || a.height_col <= 0 || a.width_col <= 0 ||
-      a.pad_h < 0 || a.pad_w < 0)
-    return fail(HF_EINVAL, "im2col_kernel: non-positive geometry");
-  if (a.n % (a.height_col * a.width_col) != 0)
-    return fail(HF_EINVAL, "im2col_kernel: n is not channels * height_col * width_col");
+  if (a.n < 0 || a.n > kMaxOffset || !extent_ok(a.height) || !extent_ok(a.width) || !extent_ok(a.kernel_h) ||
+      !extent_ok(a.kernel_w) || !extent_ok(a.stride_h) || !extent_ok(a.stride_w) || !extent_ok(a.dilation_h) ||
+      !extent_ok(a.dilation_w) || !extent_ok(a.height_col) || !extent_ok(a.width_col) || !pad_ok(a.pad_h) ||
+      !pad_ok(a.pad_w))
+    return fail(HF_EINVAL, "im2col_kernel: non-positive or oversized geometry");
+  const int64_t plane_col = a.height_col * a.width_col;  // both below 2^31
+  if (a.n % plane_col != 0) return fail(HF_EINVAL, "im2col_kernel: n is not channels * height_col * width_col");
   const int64_t hc = (a.height + 2 * a.pad_h - (a.dilation_h * (a.kernel_h - 1) + 1)) / a.stride_h + 1;
   const int64_t wc = (a.width + 2 * a.pad_w - (a.dilation_w * (a.kernel_w - 1) + 1)) / a.stride_w + 1;
   if (hc != a.height_col || wc != a.width_col)
     return fail(HF_EINVAL, "im2col_kernel: height_col/width_col do not follow from the geometry");
+  const int64_t channels = a.n / plane_col;
+  int64_t in_elems, out_elems;
+  if (!product(in_elems, {channels, a.height, a.width}) || !product(out_elems, {a.n, a.kernel_h, a.kernel_w}))
+    return fail(HF_EINVAL, "im2col_kernel: tensor sizes overflow");
   std::memcpy(p.blob, &a, sizeof a);
-  const int64_t channels = a.n / (a.height_col * a.width_col);
   const bool fast = a.kernel_h == 3 && a.kernel_w == 3 && a.stride_h == 1 && a.stride_w == 1 && a.pad_h == 1 &&
                     a.pad_w == 1 && a.dilation_h == 1 && a.dilation_w == 1 && a.width % 4 == 0 &&
-                    aligned16(a.data_im) && aligned16(a.data_col) &&
-                    channels * 9 * a.height * a.width < (int64_t)1 << 31;
+                    aligned16(a.data_im) && aligned16(a.data_col) && out_elems < (int64_t)1 << 31;
   p.hint = fast ? HINT_IM2COL_3X3_S1P1 : HINT_GENERIC;
   p.items = fast ? (unsigned long long)a.n / 4 : (unsigned long long)a.n;
   return HF_OK;
@@ -190,17 +209,23 @@ int prepare_maxpool(const hf_maxpool_args &a, Prepared &p) {
       a.pooled_width <= 0 || a.kernel_h <= 0 || a.kernel_w <= 0 || a.stride_h <= 0 || a.stride_w <= 0 ||
       a.pad_h < 0 || a.pad_w < 0 || a.dilation_h <= 0 || a.dilation_w <= 0)
     return fail(HF_EINVAL, "MaxPoolForward: non-positive geometry");
-  if ((int64_t)a.nthreads != (int64_t)a.num * a.channels * a.pooled_height * a.pooled_width)
+  int64_t out_elems, in_elems;
+  if (!product(out_elems, {a.num, a.channels, a.pooled_height, a.pooled_width}) || out_elems != (int64_t)a.nthreads)
     return fail(HF_EINVAL, "MaxPoolForward: nthreads is not num * channels * pooled_height * pooled_width");
-  if (a.pad_h * 2 > (a.kernel_h - 1) * a.dilation_h + 1 || a.pad_w * 2 > (a.kernel_w - 1) * a.dilation_w + 1)
+  if (!product(in_elems, {a.num, a.channels, a.height, a.width}))
+    return fail(HF_EINVAL, "MaxPoolForward: input size overflows");
+  const int64_t eff_h = ((int64_t)a.kernel_h - 1) * a.dilation_h + 1, eff_w = ((int64_t)a.kernel_w - 1) * a.dilation_w + 1;
+  if (eff_h >= kMaxExtent || eff_w >= kMaxExtent) return fail(HF_EINVAL, "MaxPoolForward: effective kernel size overflows");
+  if ((int64_t)a.pad_h * 2 > eff_h || (int64_t)a.pad_w * 2 > eff_w)
     return fail(HF_EINVAL, "MaxPoolForward: pad should be at most half of the effective kernel size");
-  if ((a.pooled_height - 1) * a.stride_h - a.pad_h >= a.height || (a.pooled_width - 1) * a.stride_w - a.pad_w >= a.width)
+  if (((int64_t)a.pooled_height - 1) * a.stride_h - a.pad_h >= a.height ||
+      ((int64_t)a.pooled_width - 1) * a.stride_w - a.pad_w >= a.width)
     return fail(HF_EINVAL, "MaxPoolForward: last window starts outside the input");
   std::memcpy(p.blob, &a, sizeof a);
   const bool common = a.stride_h == 2 && a.stride_w == 2 && a.dilation_h == 1 && a.dilation_w == 1 &&
-                      a.width % 4 == 0 && a.pooled_width * 2 == a.width && a.pooled_width % 2 == 0 &&
+                      a.width % 4 == 0 && (int64_t)a.pooled_width * 2 == a.width && a.pooled_width % 2 == 0 &&
                       aligned16(a.bottom_data) && aligned16(a.top_data) && aligned16(a.top_mask) &&
-                      (int64_t)a.num * a.channels * a.height * a.width < (int64_t)1 << 31;
+                      in_elems < (int64_t)1 << 31;
   p.hint = HINT_GENERIC;
   if (common && a.kernel_h == 3 && a.kernel_w == 3 && a.pad_h == 1 && a.pad_w == 1 &&
       a.pooled_height == (a.height + 2 - 3) / 2 + 1)
@@ -213,14 +238,29 @@ int prepare_maxpool(const hf_maxpool_args &a, Prepared &p) {
 }
 
 int prepare_bn(const hf_bn_stats_args &a, Prepared &p) {
+  const char *who = "batch_norm_collect_statistics_kernel: ";
   if (!a.input.data || !a.save_mean.data || !a.save_transformed_var.data)
-    return fail(HF_EINVAL, "batch_norm_collect_statistics_kernel: null data pointer");
+    return fail(HF_EINVAL, std::string(who) + "null data pointer");
   if (a.input.sizes[0] <= 0 || a.input.sizes[1] <= 0 || a.input.sizes[2] <= 0)
-    return fail(HF_EINVAL, "batch_norm_collect_statistics_kernel: empty input");
+    return fail(HF_EINVAL, std::string(who) + "empty input");
   if (a.save_mean.sizes[0] != a.input.sizes[1] || a.save_transformed_var.sizes[0] != a.input.sizes[1])
-    return fail(HF_EINVAL, "batch_norm_collect_statistics_kernel: output length is not the channel count");
-  for (int i = 0; i < 3; i++)
-    if (a.input.strides[i] < 0) return fail(HF_EINVAL, "batch_norm_collect_statistics_kernel: negative stride");
+    return fail(HF_EINVAL, std::string(who) + "output length is not the channel count");
+  // one plane's N * L elements are walked with 32-bit counters; the farthest element of the
+  // (possibly strided) input and outputs must be addressable
+  int64_t plane, reach = 0;
+  if (!extent_ok(a.input.sizes[0]) || !extent_ok(a.input.sizes[1]) || !extent_ok(a.input.sizes[2]) ||
+      !product(plane, {a.input.sizes[0], a.input.sizes[2]}) || plane >= kMaxExtent)
+    return fail(HF_EUNSUPPORTED, std::string(who) + "planes of 2^31 elements or more are not built");
+  for (int i = 0; i < 3; i++) {
+    int64_t far;
+    if (a.input.strides[i] < 0 || !product(far, {a.input.sizes[i] - 1, a.input.strides[i]}) ||
+        __builtin_add_overflow(reach, far, &reach) || reach > kMaxOffset)
+      return fail(HF_EINVAL, std::string(who) + "negative or oversized stride");
+  }
+  int64_t far;
+  if (!product(far, {a.input.sizes[1] - 1, a.save_mean.strides[0]}) ||
+      !product(far, {a.input.sizes[1] - 1, a.save_transformed_var.strides[0]}))
+    return fail(HF_EINVAL, std::string(who) + "negative or oversized output stride");
   std::memcpy(p.blob, &a, sizeof a);
   const bool fast = a.input.strides[2] == 1 && a.input.sizes[2] % 4 == 0 && a.input.strides[0] % 4 == 0 &&
                     a.input.strides[1] % 4 == 0 && aligned16(a.input.data);
@@ -236,12 +276,18 @@ int prepare_upsample(const hf_upsample_nearest_args &a, Prepared &p) {
     return fail(HF_EINVAL, "upsample_nearest2d_out_frame: empty tensor");
   if (!(a.height_scale > 0.0f) || !(a.width_scale > 0.0f))
     return fail(HF_EINVAL, "upsample_nearest2d_out_frame: scale must be positive");
+  int64_t in_elems, out_elems;
+  if (a.nc >= (size_t)kMaxExtent || a.height1 >= (size_t)kMaxExtent || a.width1 >= (size_t)kMaxExtent ||
+      a.height2 >= (size_t)kMaxExtent || a.width2 >= (size_t)kMaxExtent ||
+      !product(in_elems, {(int64_t)a.nc, (int64_t)a.height1, (int64_t)a.width1}) ||
+      !product(out_elems, {(int64_t)a.nc, (int64_t)a.height2, (int64_t)a.width2}))
+    return fail(HF_EINVAL, "upsample_nearest2d_out_frame: tensor sizes overflow");
   std::memcpy(p.blob, &a, sizeof a);
   const bool fast = a.height2 == 2 * a.height1 && a.width2 == 2 * a.width1 && a.height_scale == 0.5f &&
                     a.width_scale == 0.5f && a.width1 % 2 == 0 && aligned16(a.idata) && aligned16(a.odata) &&
-                    a.nc * a.height2 * a.width2 < (size_t)1 << 32;
+                    out_elems < (int64_t)1 << 32;
   p.hint = fast ? HINT_UP_2X : HINT_GENERIC;
-  p.items = fast ? a.nc * a.height1 * (a.width1 / 2) : a.nc * a.height2 * a.width2;
+  p.items = fast ? (unsigned long long)in_elems / 2 : (unsigned long long)out_elems;
   return HF_OK;
 }
 
@@ -252,13 +298,23 @@ int prepare_bilinear(const hf_upsample_bilinear_args &a, Prepared &p) {
     if (a.idata.sizes[i] <= 0 || a.odata.sizes[i] <= 0) return fail(HF_EINVAL, std::string(who) + "empty tensor");
   if (a.idata.sizes[0] != a.odata.sizes[0] || a.idata.sizes[1] != a.odata.sizes[1])
     return fail(HF_EINVAL, std::string(who) + "batch / channel counts of input and output differ");
-  if ((int64_t)a.n != a.odata.sizes[2] * a.odata.sizes[3])
+  int64_t total, in_total, hw;
+  if (!product(total, {a.odata.sizes[0], a.odata.sizes[1], a.odata.sizes[2], a.odata.sizes[3]}) ||
+      !product(in_total, {a.idata.sizes[0], a.idata.sizes[1], a.idata.sizes[2], a.idata.sizes[3]}) ||
+      total >= (int64_t)1 << 32 || in_total >= (int64_t)1 << 32)
+    return fail(HF_EUNSUPPORTED, std::string(who) + "tensors of 2^32 elements or more are not built");
+  if (!product(hw, {a.odata.sizes[2], a.odata.sizes[3]}) || (int64_t)a.n != hw)
     return fail(HF_EINVAL, std::string(who) + "n is not height2 * width2");
   if (!(a.rheight >= 0.0f) || !(a.rwidth >= 0.0f)) return fail(HF_EINVAL, std::string(who) + "negative scale");
-  const int64_t total = a.odata.sizes[0] * a.odata.sizes[1] * a.odata.sizes[2] * a.odata.sizes[3];
-  const int64_t in_total = a.idata.sizes[0] * a.idata.sizes[1] * a.idata.sizes[2] * a.idata.sizes[3];
-  if (total >= (int64_t)1 << 32 || in_total >= (int64_t)1 << 32)
-    return fail(HF_EUNSUPPORTED, std::string(who) + "tensors of 2^32 elements or more are not built");
+  for (const hf_accessor4 *t : {&a.idata, &a.odata}) {
+    int64_t reach = 0;
+    for (int i = 0; i < 4; i++) {
+      int64_t far;
+      if (t->strides[i] < 0 || !product(far, {t->sizes[i] - 1, t->strides[i]}) ||
+          __builtin_add_overflow(reach, far, &reach) || reach > kMaxOffset)
+        return fail(HF_EINVAL, std::string(who) + "negative or oversized stride");
+    }
+  }
   std::memcpy(p.blob, &a, sizeof a);
   auto contiguous = [](const hf_accessor4 &t) {
     return t.strides[3] == 1 && t.strides[2] == t.sizes[3] && t.strides[1] == t.sizes[2] * t.sizes[3] &&
@@ -280,13 +336,17 @@ int prepare_histc(const hf_histc_args &a, Prepared &p) {
   if (!a.a.data || !a.b.data) return fail(HF_EINVAL, "kernelHistogram1D: null data pointer");
   if (a.nbins <= 0) return fail(HF_EINVAL, "kernelHistogram1D: bins must be > 0");
   if (!(a.minvalue < a.maxvalue)) return fail(HF_EINVAL, "kernelHistogram1D: max must be larger than min");
-  if (a.total_elements < 0) return fail(HF_EINVAL, "kernelHistogram1D: negative element count");
+  if (a.total_elements < 0 || a.total_elements > kMaxOffset)
+    return fail(HF_EINVAL, "kernelHistogram1D: negative or oversized element count");
   if (a.a.dims != 1 || a.b.dims != 1)
     return fail(HF_EUNSUPPORTED, "kernelHistogram1D: only 1-D tensors are built");
   if (a.a.sizes[0] != a.nbins) return fail(HF_EINVAL, "kernelHistogram1D: output length is not nbins");
   if (a.b.sizes[0] != a.total_elements) return fail(HF_EINVAL, "kernelHistogram1D: totalElements is not the input length");
   if (a.a.strides[0] != 1) return fail(HF_EUNSUPPORTED, "kernelHistogram1D: output must be contiguous");
   if (a.nbins > 15360) return fail(HF_EUNSUPPORTED, "kernelHistogram1D: more bins than fit the LDS budget (15360)");
+  int64_t far;
+  if (a.b.strides[0] < 0 || !product(far, {a.total_elements > 0 ? a.total_elements - 1 : 0, a.b.strides[0]}))
+    return fail(HF_EINVAL, "kernelHistogram1D: negative or oversized input stride");
   std::memcpy(p.blob, &a, sizeof a);
   const bool fast = a.b.strides[0] == 1 && aligned16(a.b.data);
   // max - min a power of two (exact reciprocal): the division in the bin formula can be a multiply

@@ -396,6 +396,10 @@ def test_launch_argument_errors_never_reach_the_gpu(cfg):
     assert b"max must be larger than min" in lib.hf_last_error()
     v = cfg.plan(0, "vfuse")
     assert lib.hf_launch_fused(v._h, C.byref(a), C.byref(b), 0, None) in (L.HF_EINVAL, L.HF_EUNSUPPORTED)
+    # extents whose product wraps to zero used to divide by zero; every extent is bounded now
+    a.height_col = a.width_col = 1 << 32
+    assert lib.hf_launch_native(b"im2col_kernel", C.byref(a), 0, 0, None) == L.HF_EINVAL
+    assert b"oversized geometry" in lib.hf_last_error()
     # a grid whose thread count does not fit the bodies' 32-bit work-item counters
     a.height_col, a.width_col = 8, 8
     assert lib.hf_launch_native(b"im2col_kernel", C.byref(a), 1 << 23, 1024, None) == L.HF_EINVAL
