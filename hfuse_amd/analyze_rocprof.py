@@ -155,16 +155,17 @@ def exec_time_table(dispatches: List[Dispatch], reducer=statistics.median) -> Di
     return table
 
 
-def load_counters(paths: Iterable[str]) -> Dict[KernelKey, Dict[str, float]]:
-    """Median per dispatch of every counter, per kernel and block shape."""
-    acc: Dict[KernelKey, Dict[str, List[float]]] = defaultdict(lambda: defaultdict(list))
+def load_counters(paths: Iterable[str]) -> Dict[Tuple[KernelKey, int], Dict[str, float]]:
+    """Median per dispatch of every counter, per kernel, block shape and grid size (one kernel
+    launched at two shapes, such as max-pool in two pairs, gives two rows)."""
+    acc: Dict[Tuple[KernelKey, int], Dict[str, List[float]]] = defaultdict(lambda: defaultdict(list))
     for path in paths:
         with open(path, newline="") as f:
             for r in csv.DictReader(f):
                 p = parse_kernel_name(r["Kernel_Name"])
                 if p is None:
                     continue
-                key = KernelKey(p[0], p[1], int(r["Workgroup_Size"]))
+                key = (KernelKey(p[0], p[1], int(r["Workgroup_Size"])), int(r.get("Grid_Size", 0) or 0))
                 acc[key][r["Counter_Name"]].append(float(r["Counter_Value"]))
     return {k: {c: statistics.median(v) for c, v in cs.items()} for k, cs in acc.items()}
 
@@ -211,11 +212,16 @@ def derived_metrics(c: Dict[str, float], cus: int = 256, xcds: int = 8) -> Dict[
     return out
 
 
-def metric_table(counters: Dict[KernelKey, Dict[str, float]], cus: int = 256, xcds: int = 8):
+def metric_table(counters: Dict[Tuple[KernelKey, int], Dict[str, float]], cus: int = 256, xcds: int = 8):
     rows = []
-    for key in sorted(counters, key=lambda k: (len(k.kernels), k.kernels, TAG_ORDER.index(k.tag), k.block)):
+    shapes = defaultdict(set)
+    for key, grid in counters:
+        shapes[key].add(grid)
+    order = sorted(counters, key=lambda kg: (len(kg[0].kernels), kg[0].kernels, TAG_ORDER.index(kg[0].tag), kg[0].block, kg[1]))
+    for key, grid in order:
         name = "+".join(SHORT.get(k, k) for k in key.kernels)
-        rows.append((name, key.label(), derived_metrics(counters[key], cus, xcds)))
+        label = key.label() + (f" grid {grid}" if len(shapes[key]) > 1 else "")   # grid in work-items, as rocprofv3 reports it
+        rows.append((name, label, derived_metrics(counters[(key, grid)], cus, xcds)))
     return rows
 
 

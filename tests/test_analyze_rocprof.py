@@ -98,3 +98,10 @@ def test_metric_table(tmp_path):
     md = A.render_metric_table(rows)
     assert "| SHA256 | ST | 99.0 | 10.0 | 72.0 | 4096 |" in md and "| SHA256+Blake2B | HF@256 | 50.0 | * | 40.0 | 8192 |" in md
     assert A.agent_shape(str(p)) == (256, 8)   # no agent_info.csv beside it: MI355X
+    # the same kernel at a second grid size gets its own row, labelled with the grid
+    with open(p, "a", newline="") as f:
+        w = csv.DictWriter(f, fieldnames=cols, quoting=csv.QUOTE_NONNUMERIC)
+        w.writerow({"Dispatch_Id": 9, "Kernel_Name": sha, "Workgroup_Size": 128, "Grid_Size": 1 << 10, "VGPR_Count": 64,
+                    "Counter_Name": "SQ_WAVES", "Counter_Value": 16.0})
+    labels = [(n, t) for n, t, _ in A.metric_table(A.load_counters([str(p)]))]
+    assert labels == [("SHA256", "ST grid 1024"), ("SHA256", "ST grid 1048576"), ("SHA256+Blake2B", "HF@256")]
