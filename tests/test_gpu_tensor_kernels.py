@@ -548,3 +548,35 @@ def test_empty_work_is_a_no_op(cuda, cfg):
             sync()
             pool.check()
     assert float(out.min()) == 7.0 and float(out.max()) == 7.0
+
+
+def test_launches_can_be_captured_in_a_graph(cuda, cfg):
+    """Native and fused launches only enqueue kernels on the caller's stream (no allocation, no
+    synchronisation, no memset), so a stream capture records them; every replay must give the
+    eager result, with eager work and synchronisations between the replays."""
+    i = cfg.find_fusion("kernelHistogram1D", "batch_norm_collect_statistics_kernel")
+    j = cfg.find_fusion("im2col_kernel", "MaxPoolForward")
+    hist, bn = Histc(cuda, 100000), BnStats(cuda, 4, 9, 6, 6)
+    col, pool = Im2col(cuda, 2, 4, 12, 12), MaxPool(cuda, 2, 4, 16, 16, (3, 3), (2, 2), (1, 1))
+    up = Upsample(cuda, 2, 3, 8, 8, (16, 16))
+    p1, p2 = cfg.plan(i), cfg.plan(j)
+    p1.launch(hist.args, bn.args)          # warm-up outside the capture (first-use initialisation)
+    p2.launch(col.args, pool.args)
+    H.launch_native("upsample_nearest2d_out_frame", up.args)
+    sync()
+    side = torch.cuda.Stream()             # default priority
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.stream(side):
+        with torch.cuda.graph(graph, stream=side):
+            hist.out.zero_()               # a fill kernel, not a memset node
+            p1.launch(hist.args, bn.args)
+            p2.launch(col.args, pool.args)
+            H.launch_native("upsample_nearest2d_out_frame", up.args)
+    for t in (hist, bn, col, pool, up):    # the warm-up results; check() also scrubs the outputs
+        t.check()
+    hist.out.fill_(5.0)                    # the captured fill kernel has to clear this
+    for replay in range(3):
+        graph.replay()
+        sync()
+        for t in (hist, bn, col, pool, up):
+            t.check()                      # eager copies, comparisons and fills between the replays
