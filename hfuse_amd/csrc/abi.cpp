@@ -198,7 +198,14 @@ int prepare_im2col(const hf_im2col_args &a, Prepared &p) {
   const bool fast = a.kernel_h == 3 && a.kernel_w == 3 && a.stride_h == 1 && a.stride_w == 1 && a.pad_h == 1 &&
                     a.pad_w == 1 && a.dilation_h == 1 && a.dilation_w == 1 && a.width % 4 == 0 &&
                     aligned16(a.data_im) && aligned16(a.data_col) && out_elems < (int64_t)1 << 31;
-  p.hint = fast ? HINT_IM2COL_3X3_S1P1 : HINT_GENERIC;
+  // 32-bit index arithmetic in the general loop: every element offset, and the window reach
+  // (effective kernel + padding) times the row length, stays below 2^31
+  const int64_t lim = (int64_t)1 << 31;
+  const bool idx32 = in_elems < lim && out_elems < lim &&
+                     (a.dilation_h * (a.kernel_h - 1) + 1 + a.pad_h + a.height) * a.width < lim &&
+                     a.dilation_w * (a.kernel_w - 1) + 1 + a.pad_w + a.width < lim &&
+                     a.height_col * a.stride_h < lim && a.width_col * a.stride_w < lim;
+  p.hint = fast ? HINT_IM2COL_3X3_S1P1 : idx32 ? HINT_IDX32 : HINT_GENERIC;
   p.items = fast ? (unsigned long long)a.n / 4 : (unsigned long long)a.n;
   return HF_OK;
 }
@@ -226,14 +233,15 @@ int prepare_maxpool(const hf_maxpool_args &a, Prepared &p) {
                       a.width % 4 == 0 && (int64_t)a.pooled_width * 2 == a.width && a.pooled_width % 2 == 0 &&
                       aligned16(a.bottom_data) && aligned16(a.top_data) && aligned16(a.top_mask) &&
                       in_elems < (int64_t)1 << 31;
-  p.hint = HINT_GENERIC;
+  p.hint = (in_elems < (int64_t)1 << 31 && out_elems < (int64_t)1 << 31) ? HINT_IDX32 : HINT_GENERIC;
   if (common && a.kernel_h == 3 && a.kernel_w == 3 && a.pad_h == 1 && a.pad_w == 1 &&
       a.pooled_height == (a.height + 2 - 3) / 2 + 1)
     p.hint = HINT_POOL_K3S2P1;
   if (common && a.kernel_h == 2 && a.kernel_w == 2 && a.pad_h == 0 && a.pad_w == 0 &&
       a.pooled_height == (a.height - 2) / 2 + 1)
     p.hint = HINT_POOL_K2S2P0;
-  p.items = p.hint ? (unsigned long long)a.nthreads / 2 : (unsigned long long)a.nthreads;
+  p.items = (p.hint == HINT_POOL_K3S2P1 || p.hint == HINT_POOL_K2S2P0) ? (unsigned long long)a.nthreads / 2
+                                                                         : (unsigned long long)a.nthreads;
   return HF_OK;
 }
 
@@ -286,7 +294,7 @@ int prepare_upsample(const hf_upsample_nearest_args &a, Prepared &p) {
   const bool fast = a.height2 == 2 * a.height1 && a.width2 == 2 * a.width1 && a.height_scale == 0.5f &&
                     a.width_scale == 0.5f && a.width1 % 2 == 0 && aligned16(a.idata) && aligned16(a.odata) &&
                     out_elems < (int64_t)1 << 32;
-  p.hint = fast ? HINT_UP_2X : HINT_GENERIC;
+  p.hint = fast ? HINT_UP_2X : (in_elems < (int64_t)1 << 31 && out_elems < (int64_t)1 << 31) ? HINT_IDX32 : HINT_GENERIC;
   p.items = fast ? (unsigned long long)in_elems / 2 : (unsigned long long)out_elems;
   return HF_OK;
 }
@@ -348,12 +356,15 @@ int prepare_histc(const hf_histc_args &a, Prepared &p) {
   if (a.b.strides[0] < 0 || !product(far, {a.total_elements > 0 ? a.total_elements - 1 : 0, a.b.strides[0]}))
     return fail(HF_EINVAL, "kernelHistogram1D: negative or oversized input stride");
   std::memcpy(p.blob, &a, sizeof a);
-  const bool fast = a.b.strides[0] == 1 && aligned16(a.b.data);
+  // contiguous input: 16-byte loads from the first aligned element on; the up to three elements
+  // before it (HINT_HIST_HEAD bits) and the tail go through scalar loads
+  const bool fast = a.b.strides[0] == 1 && (reinterpret_cast<uintptr_t>(a.b.data) & 3u) == 0;
+  const unsigned head = fast ? (unsigned)(((16u - (reinterpret_cast<uintptr_t>(a.b.data) & 15u)) & 15u) >> 2) : 0u;
   // max - min a power of two (exact reciprocal): the division in the bin formula can be a multiply
   int exp2 = 0;
   const float range = a.maxvalue - a.minvalue;
   const bool pow2 = std::frexp(range, &exp2) == 0.5f && exp2 > -100 && exp2 < 100;
-  p.hint = (fast ? HINT_HIST_VEC4 : HINT_GENERIC) | (pow2 ? HINT_HIST_POW2 : 0);
+  p.hint = (fast ? HINT_HIST_VEC4 : HINT_GENERIC) | (pow2 ? HINT_HIST_POW2 : 0) | (head << HINT_HIST_HEAD_SHIFT);
   p.lds = (unsigned)a.nbins * 4u;
   p.items = fast ? (unsigned long long)(a.total_elements + 3) / 4 : (unsigned long long)a.total_elements;
   return HF_OK;

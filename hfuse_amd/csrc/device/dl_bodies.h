@@ -13,7 +13,9 @@
 namespace hfuse {
 
 // Hints (0 always means the general path).
-enum { HINT_GENERIC = 0, HINT_IM2COL_3X3_S1P1 = 1, HINT_POOL_K3S2P1 = 1, HINT_POOL_K2S2P0 = 2, HINT_UP_2X = 1, HINT_BN_VEC4 = 1, HINT_HIST_VEC4 = 1, HINT_HIST_POW2 = 2, HINT_BILINEAR_VEC4 = 1, HINT_BILINEAR_2X = 2 };
+enum { HINT_GENERIC = 0, HINT_IM2COL_3X3_S1P1 = 1, HINT_POOL_K3S2P1 = 1, HINT_POOL_K2S2P0 = 2, HINT_UP_2X = 1, HINT_BN_VEC4 = 1, HINT_HIST_VEC4 = 1, HINT_HIST_POW2 = 2, HINT_HIST_HEAD_SHIFT = 4 /* bits 4-5: elements before the first 16-byte boundary */, HINT_BILINEAR_VEC4 = 1, HINT_BILINEAR_2X = 2,
+       // general path with 32-bit index arithmetic: every tensor of the call has fewer than 2^31 elements
+       HINT_IDX32 = 0x100 };
 
 __device__ __forceinline__ f32x4 ld4(const float *p) { return *reinterpret_cast<const f32x4 *>(p); }
 
@@ -50,24 +52,33 @@ struct Im2colBody {
       vec4_3x3(a, sb);
       return;
     }
-    const int64_t stride = (int64_t)sb.gstride();
-    const int64_t plane_col = a.height_col * a.width_col;
-    for (int64_t index = (int64_t)sb.gtid(); index < a.n; index += stride) {
-      const int64_t w_out = index % a.width_col;
-      const int64_t idx = index / a.width_col;
-      const int64_t h_out = idx % a.height_col;
-      const int64_t channel_in = idx / a.height_col;
-      const int64_t channel_out = channel_in * a.kernel_h * a.kernel_w;
-      const int64_t h_in = h_out * a.stride_h - a.pad_h;
-      const int64_t w_in = w_out * a.stride_w - a.pad_w;
-      float *col = a.data_col + (channel_out * a.height_col + h_out) * a.width_col + w_out;
-      const float *im = a.data_im + (channel_in * a.height + h_in) * a.width + w_in;
-      for (int64_t i = 0; i < a.kernel_h; ++i) {
-        for (int64_t j = 0; j < a.kernel_w; ++j) {
-          const int64_t h = h_in + i * a.dilation_h, w = w_in + j * a.dilation_w;
-          *col = (h >= 0 && w >= 0 && h < a.height && w < a.width)
-                     ? im[i * a.dilation_h * a.width + j * a.dilation_w]
-                     : 0.0f;
+    if (hint == HINT_IDX32) general<unsigned, int>(a, sb);
+    else general<int64_t, int64_t>(a, sb);
+  }
+
+  // The original per-element loop, any geometry.  I indexes work items and elements (64-bit
+  // division is a long instruction sequence on this part, so tensors below 2^31 elements use
+  // 32-bit indices), S is the signed type of image coordinates.
+  template <class I, class S, class SB>
+  static __device__ __forceinline__ void general(const Args &a, SB &sb) {
+    const I stride = (I)sb.gstride(), n = (I)a.n;
+    const I width_col = (I)a.width_col, height_col = (I)a.height_col, plane_col = height_col * width_col;
+    const I kh = (I)a.kernel_h, kw = (I)a.kernel_w;
+    const S height = (S)a.height, width = (S)a.width, dil_h = (S)a.dilation_h, dil_w = (S)a.dilation_w;
+    for (I index = (I)sb.gtid(); index < n; index += stride) {
+      const I w_out = index % width_col;
+      const I idx = index / width_col;
+      const I h_out = idx % height_col;
+      const I channel_in = idx / height_col;
+      const I channel_out = channel_in * kh * kw;
+      const S h_in = (S)h_out * (S)a.stride_h - (S)a.pad_h;
+      const S w_in = (S)w_out * (S)a.stride_w - (S)a.pad_w;
+      float *col = a.data_col + (size_t)((channel_out * height_col + h_out) * width_col + w_out);
+      const float *im = a.data_im + (ptrdiff_t)((S)channel_in * height + h_in) * (ptrdiff_t)width + (ptrdiff_t)w_in;
+      for (I i = 0; i < kh; ++i) {
+        for (I j = 0; j < kw; ++j) {
+          const S h = h_in + (S)i * dil_h, w = w_in + (S)j * dil_w;
+          *col = (h >= 0 && w >= 0 && h < height && w < width) ? im[(ptrdiff_t)((S)i * dil_h * width + (S)j * dil_w)] : 0.0f;
           col += plane_col;
         }
       }
@@ -142,12 +153,22 @@ struct MaxPoolBody {
   static __device__ void run(const Args &a, SB &sb, unsigned char *, unsigned hint) {
     if (hint == HINT_POOL_K3S2P1) { vec2_s2<3, 1>(a, sb); return; }
     if (hint == HINT_POOL_K2S2P0) { vec2_s2<2, 0>(a, sb); return; }
-    const int64_t stride = (int64_t)sb.gstride();
-    for (int64_t index = (int64_t)sb.gtid(); index < a.nthreads; index += stride) {
-      const int pw = (int)(index % a.pooled_width);
-      const int ph = (int)((index / a.pooled_width) % a.pooled_height);
-      const int c = (int)((index / a.pooled_width / a.pooled_height) % a.channels);
-      const int n = (int)(index / a.pooled_width / a.pooled_height / a.channels);
+    if (hint == HINT_IDX32) general<unsigned>(a, sb);
+    else general<int64_t>(a, sb);
+  }
+
+  // The original loop: any window, stride, padding and dilation.  I is the index type
+  // (32-bit when input and output have fewer than 2^31 elements).
+  template <class I, class SB>
+  static __device__ __forceinline__ void general(const Args &a, SB &sb) {
+    const I stride = (I)sb.gstride(), n = (I)a.nthreads;
+    const I pw_n = (I)a.pooled_width, ph_n = (I)a.pooled_height, ch_n = (I)a.channels;
+    for (I index = (I)sb.gtid(); index < n; index += stride) {
+      const I t0 = index / pw_n, t1 = t0 / ph_n;
+      const int pw = (int)(index - t0 * pw_n);
+      const int ph = (int)(t0 - t1 * ph_n);
+      const I nn = t1 / ch_n;
+      const int c = (int)(t1 - nn * ch_n);
       int hstart = ph * a.stride_h - a.pad_h;
       int wstart = pw * a.stride_w - a.pad_w;
       const int hend = min(hstart + (a.kernel_h - 1) * a.dilation_h + 1, a.height);
@@ -156,7 +177,7 @@ struct MaxPoolBody {
       while (wstart < 0) wstart += a.dilation_w;
       float maxval = -INFINITY;
       int maxidx = hstart * a.width + wstart;
-      const float *plane = a.bottom_data + ((int64_t)n * a.channels + c) * a.height * a.width;
+      const float *plane = a.bottom_data + (size_t)((nn * ch_n + (I)c) * (I)a.height) * (size_t)a.width;
       for (int h = hstart; h < hend; h += a.dilation_h)
         for (int w = wstart; w < wend; w += a.dilation_w) {
           const float v = plane[h * a.width + w];
@@ -293,15 +314,24 @@ struct UpsampleNearestBody {
       }
       return;
     }
-    const size_t total = a.nc * a.height2 * a.width2;
-    const size_t stride = (size_t)sb.gstride();
-    for (size_t index = (size_t)sb.gtid(); index < total; index += stride) {
-      const size_t x2 = index % a.width2;
-      const size_t y2 = (index / a.width2) % a.height2;
-      const size_t c = index / a.width2 / a.height2;
+    if (hint == HINT_IDX32) general<unsigned>(a, sb);
+    else general<size_t>(a, sb);
+  }
+
+  // The original per-pixel loop, any sizes and scales: src = min(floor(dst * scale), in - 1).
+  template <class I, class SB>
+  static __device__ __forceinline__ void general(const Args &a, SB &sb) {
+    const I w2 = (I)a.width2, h2 = (I)a.height2, w1 = (I)a.width1, h1 = (I)a.height1;
+    const I total = (I)a.nc * h2 * w2;
+    const I stride = (I)sb.gstride();
+    for (I index = (I)sb.gtid(); index < total; index += stride) {
+      const I t = index / w2;
+      const I x2 = index - t * w2;
+      const I c = t / h2;
+      const I y2 = t - c * h2;
       const int y1 = min((int)floorf((float)y2 * a.height_scale), (int)a.height1 - 1);
       const int x1 = min((int)floorf((float)x2 * a.width_scale), (int)a.width1 - 1);
-      a.odata[index] = a.idata[(c * a.height1 + y1) * a.width1 + x1];
+      a.odata[index] = a.idata[(c * h1 + (I)y1) * w1 + (I)x1];
     }
   }
 };
@@ -661,7 +691,13 @@ struct HistcBody {
       count<POW2>(bins, v.w, lo, hi, fn, range, inv_range, nbins);
     };
     if (hint & HINT_HIST_VEC4) {
-      const int64_t n4 = total >> 2;
+      // `head` elements (0..3) precede the first 16-byte boundary; block 0 counts them and the
+      // tail with scalar loads, everyone streams the aligned middle.
+      const int64_t head = min((int64_t)((hint >> HINT_HIST_HEAD_SHIFT) & 3u), total);
+      if (sb.bid == 0 && (int64_t)sb.tid < head) count<POW2>(bins, b[sb.tid], lo, hi, fn, range, inv_range, nbins);
+      b += head;
+      const int64_t rest = total - head;
+      const int64_t n4 = rest >> 2;
       const int64_t stride = (int64_t)sb.gstride();
       int64_t i = (int64_t)sb.gtid();
       // several 16-byte loads in flight per lane before the dependent LDS atomics
@@ -677,7 +713,7 @@ struct HistcBody {
       }
       for (; i < n4; i += stride) count4(ld4(b + i * 4));
       if (sb.bid == 0)
-        for (int64_t k = (n4 << 2) + sb.tid; k < total; k += sb.nthreads)
+        for (int64_t k = (n4 << 2) + sb.tid; k < rest; k += sb.nthreads)
           count<POW2>(bins, b[k], lo, hi, fn, range, inv_range, nbins);
     } else {
       const int64_t stride = (int64_t)sb.gstride();

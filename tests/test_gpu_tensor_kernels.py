@@ -312,6 +312,19 @@ def test_histc(cuda, n, nbins, lo, hi):
     t.check()
 
 
+@pytest.mark.parametrize("offset", [1, 2, 3])
+@pytest.mark.parametrize("n", [1, 2, 3, 5, 4099, 100001])
+def test_histc_unaligned_input(cuda, offset, n):
+    """A contiguous input that starts 4, 8 or 12 bytes past a 16-byte boundary still streams with
+    16-byte loads; the elements before the boundary and the tail are counted by scalar loads."""
+    x = uniform((n + offset,), 31 + n, 0.0, 1.0)
+    xd = x.to(cuda)
+    out = torch.zeros(64, device=cuda)
+    H.launch_native("kernelHistogram1D", H.histc_args(xd[offset:], out, 64, 0.0, 1.0))
+    sync()
+    assert np.array_equal(out.cpu().numpy(), O.histc(x[offset:].numpy(), 64, 0.0, 1.0))
+
+
 def test_histc_out_of_range_and_accumulation(cuda):
     x = torch.tensor([-0.5, 0.0, 0.999, 1.0, 1.5, float("nan"), 0.3, 0.3])
     t = Histc(cuda, 8, 4, 0.0, 1.0, x=x)
@@ -580,3 +593,43 @@ def test_launches_can_be_captured_in_a_graph(cuda, cfg):
         sync()
         for t in (hist, bn, col, pool, up):
             t.check()                      # eager copies, comparisons and fills between the replays
+
+
+# ------------------------------------------------------------------ sizes at and beyond 2^31 elements
+# The general loops use 32-bit indices below 2^31 elements and 64-bit ones from there on.  These
+# cases sit above the limit; the expected values come from PyTorch's own GPU operators (at these
+# sizes a CPU run of the oracle would take minutes), so they are cross-checks, not oracle parity.
+def test_upsample_nearest_beyond_2_31_elements(cuda):
+    x = torch.rand((1 << 13, 1 << 6, 1 << 10), device=cuda)          # 2^29 elements, 2 GiB
+    out = torch.empty((1 << 13, 1 << 6, 1 << 12), device=cuda)       # 2^31 elements, 8 GiB
+    a = H.upsample_nearest_args(x.unsqueeze(0), out.unsqueeze(0))
+    H.launch_native("upsample_nearest2d_out_frame", a)
+    sync()
+    for lo in range(0, 1 << 13, 1 << 10):                            # closed form: out[.., x] = in[.., x // 4]
+        assert torch.equal(out[lo:lo + (1 << 10)], x[lo:lo + (1 << 10)].repeat_interleave(4, dim=-1))
+    del x, out
+    torch.cuda.empty_cache()
+
+
+def test_maxpool_beyond_2_31_elements(cuda):
+    x = torch.rand((8, 1 << 10, 512, 512), device=cuda)              # 2^31 elements, 8 GiB
+    val = torch.empty((8, 1 << 10, 256, 256), device=cuda)
+    idx = torch.empty((8, 1 << 10, 256, 256), dtype=torch.int64, device=cuda)
+    H.launch_native("MaxPoolForward", H.maxpool_args(x, val, idx, (2, 2), (2, 2), (0, 0)))
+    sync()
+    for n in range(8):
+        tv, ti = torch.nn.functional.max_pool2d(x[n], (2, 2), (2, 2), 0, return_indices=True)
+        assert torch.equal(val[n], tv) and torch.equal(idx[n], ti)
+    del x, val, idx
+    torch.cuda.empty_cache()
+
+
+def test_im2col_beyond_2_31_elements(cuda):
+    x = torch.rand((64, 64, 256, 256), device=cuda)                  # 2^28 elements; 9 x that = 2.4e9 columns
+    col = torch.empty((64, 576, 65536), device=cuda)
+    H.launch_native("im2col_kernel", H.im2col_args(x, col))
+    sync()
+    for n in range(0, 64, 8):
+        assert torch.equal(col[n:n + 8], torch.nn.functional.unfold(x[n:n + 8], 3, padding=1))
+    del x, col
+    torch.cuda.empty_cache()
