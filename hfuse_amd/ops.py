@@ -11,6 +11,9 @@ order).  Results are the op's outputs:
     pooled, indices = ops.run(ops.max_pool2d(x, 3, 2, 1))
     (cols,), (pooled, indices) = ops.run_fused(ops.im2col(img, 3, padding=1), ops.max_pool2d(x, 3, 2, 1))
 
+The nonce searches have the same shape: `sha256d_search`, `sia_blake2b_search`, `blake2b_search`
+and `ethash_search` upload a job's constants and return an op; `hits(op)` reads the found nonces.
+
 Tensors are float32 CUDA tensors (this build's kernels are the float instantiations the
 reference fused); inputs are made contiguous where the original operator does so.  torch is used
 for allocation and streams only; every launch goes through the C-ABI.
@@ -133,6 +136,54 @@ def histc(x, bins: int = 100, min: float = 0.0, max: float = 0.0) -> Op:
     return Op("kernelHistogram1D", H.histc_args(flat, out, int(bins), lo, hi), (out,), (flat, out))
 
 
+# ------------------------------------------------------------------ nonce searches
+# The miners' host loop: constants of a search (header, target, DAG) are uploaded once per
+# job, then a launch scans `count` nonces from `start` and appends its hits to a result record.
+# The constants are per process, like the __constant__ symbols of the original kernels, so one
+# job per kind of search is live at a time.  `hits(op)` reads the record back (it synchronises).
+
+@dataclass
+class SearchOp(Op):
+    grid: int = 0          # ethash only: the launch grid fixes the nonce count (grid * 128)
+
+
+def sha256d_search(header: bytes, target64: int, start: int, count: int) -> SearchOp:
+    """Nonces in [start, start+count) (mod 2^32) whose SHA-256d of the 80-byte header, read as a
+    little-endian 256-bit number, has its top 64 bits <= target64."""
+    H.sha256d_set_block(header, target64)
+    res = H.new_search_results()
+    return SearchOp("sha256d_gpu_hash_shared", H.sha256d_args(res, count, start), (res,), (res,))
+
+
+def sia_blake2b_search(header: bytes, target64: int, start: int, count: int) -> SearchOp:
+    """Sia layout: 8-byte nonce at offset 32 of the 80-byte header, Blake2b-256, first digest word (big-endian) <= target64."""
+    H.sia_blake2b_set_block(header)
+    res = H.new_search_results()
+    return SearchOp("sia_blake2b_gpu_hash", H.blake2b_args(res, count, start, target64), (res,), (res,))
+
+
+def blake2b_search(header: bytes, target64: int, start: int, count: int) -> SearchOp:
+    """ccminer layout: 4-byte nonce at offset 76 of the 80-byte header."""
+    H.blake2b_set_block(header)
+    res = H.new_search_results()
+    return SearchOp("blake2b_gpu_hash", H.blake2b_args(res, count, start, target64), (res,), (res,))
+
+
+def ethash_search(dag, dag_items: int, header: bytes, target64: int, start: int, count: int) -> SearchOp:
+    """Ethash hashimoto over a resident DAG of `dag_items` 128-byte items; `count` is rounded up
+    to a multiple of 128 (the original's grid * block nonces)."""
+    H.ethash_set_constants(dag, dag_items, header, target64)
+    res = H.new_search_results()
+    return SearchOp("ethash_search", H.ethash_args(res, start), (res,), (res, dag), grid=(int(count) + 127) // 128)
+
+
+def hits(op: SearchOp):
+    """-> (number found, [(nonce, digest bytes, mix bytes)] sorted by nonce, at most 64 kept)."""
+    import torch
+    torch.cuda.synchronize()
+    return H.read_search_results(op.outputs[0])
+
+
 _default_cfg: Optional[H.Config] = None
 
 
@@ -148,7 +199,7 @@ def _config(cfg: Optional[H.Config]) -> H.Config:
 
 def run(op: Op, stream=None):
     """Launch one original kernel; returns its outputs (a tuple)."""
-    H.launch_native(op.kernel, op.args, stream=stream)
+    H.launch_native(op.kernel, op.args, getattr(op, "grid", 0), 0, stream=stream)
     return op.outputs
 
 
@@ -158,10 +209,12 @@ def run_fused(op1: Op, op2: Op, cfg: Optional[H.Config] = None, preset: str = "h
     The pair is looked up in the fusion list of `cfg` (default: the shipped list) in either
     order; a pair the list does not name raises KeyError."""
     c = _config(cfg)
+    grid = max(getattr(op1, "grid", 0), getattr(op2, "grid", 0))     # ethash's exact grid, 0 otherwise
     try:
-        plan = c.plan(c.find_fusion(op1.kernel, op2.kernel), preset)
-        plan.launch(op1.args, op2.args, stream=stream)
+        first, second = op1, op2
+        index = c.find_fusion(op1.kernel, op2.kernel)
     except KeyError:
-        plan = c.plan(c.find_fusion(op2.kernel, op1.kernel), preset)
-        plan.launch(op2.args, op1.args, stream=stream)
+        first, second = op2, op1
+        index = c.find_fusion(op2.kernel, op1.kernel)
+    c.plan(index, preset).launch(first.args, second.args, grid_blocks=grid, stream=stream)
     return op1.outputs, op2.outputs

@@ -71,3 +71,38 @@ def test_fused_operators_in_either_order(cuda):
     assert torch.equal(up.cpu(), F.interpolate(x, scale_factor=2, mode="nearest"))
     with pytest.raises(KeyError):
         ops.run_fused(ops.upsample_nearest2d(xd, scale_factor=2), ops.upsample_bilinear2d(xd, scale_factor=2))
+
+
+@pytest.mark.gpu
+def test_search_operators(cuda):
+    from oracle import oracle as O
+    easy = (1 << 52) - 1
+    hdr_a, hdr_b = O.seeded_bytes(80, 91), O.seeded_bytes(80, 92)
+    a = ops.sha256d_search(hdr_a, easy, 1000, 1 << 15)
+    ops.run(a)
+    found, got = ops.hits(a)
+    want = O.sha256d_search(hdr_a, 1000, 1 << 15, easy)
+    assert found == want[0] > 0 and [g[0] for g in got] == [h.nonce for h in want[1]]
+    assert all(g[1] == O.sha256d_80(hdr_a, g[0]) for g in got)
+    # fused with the Sia search, named in the list as (sha256d, sia): pass them the other way round
+    a, b = ops.sha256d_search(hdr_a, easy, 0, 1 << 14), ops.sia_blake2b_search(hdr_b, easy, 0, 1 << 15)
+    ops.run_fused(b, a)
+    fa, ga = ops.hits(a)
+    fb, gb = ops.hits(b)
+    assert fa == O.sha256d_search(hdr_a, 0, 1 << 14, easy)[0] > 0 and fb == O.sia_search(hdr_b, 0, 1 << 15, easy)[0] > 0
+    assert all(g[1] == O.sia_blake2b_80(hdr_b, g[0]) for g in gb)
+    # ethash over a small synthetic DAG, alone and next to blake2b
+    from hfuse_amd import launcher as H
+    n_items, seed = 1 << 12, 0x48467573
+    dag = torch.empty(n_items * 32, dtype=torch.int32, device=cuda)
+    H.fill_splitmix64(dag, seed)
+    hdr = O.seeded_bytes(32, 93)
+    target = (1 << 56) - 1
+    want_n, want_h = O.ethash_search(None, seed, n_items, hdr, 0, 4096, target)
+    e = ops.ethash_search(dag, n_items, hdr, target, 0, 4096)
+    ops.run(e)
+    assert ops.hits(e) == (want_n, [(h.nonce, h.digest_bytes(), h.mix_bytes()) for h in want_h]) and want_n > 0
+    e, b = ops.ethash_search(dag, n_items, hdr, target, 0, 4096), ops.sia_blake2b_search(hdr_b, easy, 0, 1 << 15)
+    ops.run_fused(e, b)
+    assert ops.hits(e) == (want_n, [(h.nonce, h.digest_bytes(), h.mix_bytes()) for h in want_h])
+    assert ops.hits(b)[0] == fb
