@@ -27,6 +27,10 @@
  *   im2col, max_pool, upsample, histc, bn stats : PyTorch CPU ops, closed
  *                       forms (centre tap of im2col is the image, out[h][w] =
  *                       in[h/2][w/2], sum of bins = n) and brute force.
+ *   bilinear upsample : PyTorch CPU interpolate(mode="bilinear") to rounding
+ *                       (2 ulp at power-of-two ratios, a few ulp of the source
+ *                       index otherwise) and closed forms (same size is a copy,
+ *                       constants, kept corners, the 0.25 / 0.75 weights of 2x).
  *   SHA-256d          : hashlib, NIST "abc", Bitcoin genesis header.
  *   BLAKE2b           : hashlib.blake2b, RFC 7693 appendix A.
  *   Keccak            : hashlib.sha3_* (pad 0x06) and the Keccak-256/512 empty
@@ -42,7 +46,10 @@
  *     orc_*_search are this build's own;
  *   - PyTorch 1.4's histogram bin rounding for a general (min, max, nbins); for
  *     power-of-two ranges such as (0, 1, 1024) the formula is exact and is
- *     pinned against torch.histc.
+ *     pinned against torch.histc;
+ *   - the bits of PyTorch 1.4's CUDA bilinear kernel: nvcc contracts some of its
+ *     products and sums into fused multiply-adds, this restatement rounds every
+ *     one of them (the interpolant itself is pinned as above).
  */
 #include <math.h>
 #include <stdint.h>
