@@ -63,10 +63,18 @@ struct Parser {
     return false;
   }
 
+  // The two documents nest four levels deep; a bound keeps a crafted file from exhausting
+  // the stack through the mutual recursion of blocks, sequences and maps.
+  static constexpr int kMaxDepth = 32;
+  int depth = 0;
+
   bool parse_block(int indent, YamlNode &out) {
     if (pos >= lines.size()) return true;
-    if (is_seq_item(lines[pos].text)) return parse_seq(indent, out);
-    return parse_map(indent, out);
+    if (depth >= kMaxDepth) return fail(lines[pos].no, "nesting deeper than 32 levels");
+    depth++;
+    const bool ok = is_seq_item(lines[pos].text) ? parse_seq(indent, out) : parse_map(indent, out);
+    depth--;
+    return ok;
   }
 
   bool parse_seq(int indent, YamlNode &out) {

@@ -423,3 +423,15 @@ def test_header_symbols_are_all_exported():
     for name in declared:
         assert hasattr(lib, name), name
     assert lib.hf_version() >= 100
+
+
+def test_deep_nesting_is_refused_not_followed():
+    """A file nested thousands of levels deep must come back as a parse error (bounded recursion)."""
+    deep = "".join(" " * i + f"k{i}:\n" for i in range(5000)) + " " * 5000 + "v: 1\n"
+    with pytest.raises(hfuse_amd.HfuseError) as e:
+        Config(None, deep)
+    assert e.value.code == L.HF_EPARSE and "nesting" in e.value.message
+    seqs = "".join(" " * i + "-\n" for i in range(5000)) + " " * 5000 + "- x\n"
+    with pytest.raises(hfuse_amd.HfuseError) as e:
+        Config(seqs, KERNELS_MAP)
+    assert e.value.code == L.HF_EPARSE
