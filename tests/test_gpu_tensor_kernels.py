@@ -636,3 +636,40 @@ def test_im2col_beyond_2_31_elements(cuda):
         assert torch.equal(col[n:n + 8], torch.nn.functional.unfold(x[n:n + 8], 3, padding=1))
     del x, col
     torch.cuda.empty_cache()
+
+
+def test_two_host_threads_on_their_own_streams(cuda, cfg):
+    """The C-ABI is thread-compatible: one plan per thread, launches on the thread's own stream
+    (ctypes drops the GIL during a call, so the two threads really overlap in the library)."""
+    import threading
+    errors = []
+
+    def worker(seed, fusion, make_a, make_b):
+        try:
+            stream = torch.cuda.Stream()
+            with torch.cuda.stream(stream):
+                plan = cfg.plan(fusion)
+                for rep in range(20):
+                    a, b = make_a(seed + rep), make_b(seed + rep)
+                    plan.launch(a.args, b.args, stream=stream)
+                    H.launch_native("upsample_nearest2d_out_frame", up[seed % 2].args, stream=stream)
+                    stream.synchronize()
+                    a.check()
+                    b.check()
+        except Exception as e:  # surfaced in the main thread below
+            errors.append(e)
+
+    up = [Upsample(cuda, 2, 3, 8, 8, (16, 16), seed=40), Upsample(cuda, 2, 3, 8, 8, (16, 16), seed=41)]
+    i = cfg.find_fusion("im2col_kernel", "MaxPoolForward")
+    j = cfg.find_fusion("kernelHistogram1D", "batch_norm_collect_statistics_kernel")
+    t1 = threading.Thread(target=worker, args=(100, i, lambda s: Im2col(cuda, 2, 4, 12, 12, seed=s),
+                                               lambda s: MaxPool(cuda, 2, 4, 16, 16, (3, 3), (2, 2), (1, 1), seed=s)))
+    t2 = threading.Thread(target=worker, args=(201, j, lambda s: Histc(cuda, 50000, seed=s), lambda s: BnStats(cuda, 4, 9, 6, 6, seed=s)))
+    t1.start()
+    t2.start()
+    t1.join()
+    t2.join()
+    assert not errors, errors
+    sync()
+    for u in up:
+        u.check()
