@@ -328,6 +328,25 @@ def test_histc_unaligned_input(cuda, offset, n):
     assert np.array_equal(out.cpu().numpy(), O.histc(x[offset:].numpy(), 64, 0.0, 1.0))
 
 
+@pytest.mark.parametrize("nbins,lo,hi", [(1000, 0.0, 3.0), (7, -0.7, 0.0), (15360, 0.0, 10.0), (1024, 0.1, 0.9),
+                                         (100, -5.0, 123.0), (3, 1e-3, 1e3), (1024, 0.0, 1.0)])
+def test_histc_bin_edges_with_any_range(cuda, nbins, lo, hi):
+    """Ranges whose width is not a power of two go through the real fp32 division of the bin
+    formula.  The inputs sit on and one ulp either side of every bin edge (where the rounding
+    of (v - lo) * nbins / (hi - lo) decides the bin) plus uniform draws."""
+    k = np.arange(nbins + 1, dtype=np.float64)
+    edges = (lo + k * (hi - lo) / nbins).astype(np.float32)
+    parts = [edges, np.nextafter(edges, np.float32(np.inf)), np.nextafter(edges, np.float32(-np.inf)),
+             np.nextafter(np.nextafter(edges, np.float32(np.inf)), np.float32(np.inf)),
+             uniform((50000,), 77, lo, hi).numpy()]
+    x = torch.from_numpy(np.concatenate(parts).astype(np.float32))
+    t = Histc(cuda, x.numel(), nbins, lo, hi, x=x)
+    H.launch_native("kernelHistogram1D", t.args)
+    sync()
+    got = t.out.cpu().numpy()
+    assert np.array_equal(got, O.histc(x.numpy(), nbins, lo, hi))
+
+
 def test_histc_out_of_range_and_accumulation(cuda):
     x = torch.tensor([-0.5, 0.0, 0.999, 1.0, 1.5, float("nan"), 0.3, 0.3])
     t = Histc(cuda, 8, 4, 0.0, 1.0, x=x)
