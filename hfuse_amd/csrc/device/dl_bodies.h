@@ -659,10 +659,25 @@ struct HistcBody {
   // multiplication by its (exact) reciprocal and the IEEE division sequence is not needed.
   template <bool POW2>
   static __device__ __forceinline__ void count(unsigned *bins, float v, float lo, float hi, float scale_n, float range,
-                                               float inv_range, int nbins) {
+                                               float inv_range, float inv_lo, float inv_hi, int nbins) {
     if (v >= lo && v <= hi) {
       const float t = (v - lo) * scale_n;
-      int bin = (int)(POW2 ? t * inv_range : t / range);
+      int bin;
+      if constexpr (POW2) {
+        bin = (int)(t * inv_range);
+      } else {
+        // (int)(t / range) without the division where that is safe.  t times two reciprocals that
+        // bracket 1 / range by a relative 2^-21 brackets the correctly rounded quotient; when both
+        // products truncate to the same integer so does the quotient.  Only a wavefront in which some
+        // lane's products disagree does the IEEE division (its reciprocal sequence runs at a quarter
+        // of the multiply rate); the empty asm keeps the compiler from hoisting it out of the branch.
+        bin = (int)(t * inv_lo);
+        const bool unsure = bin != (int)(t * inv_hi);
+        if (__builtin_amdgcn_ballot_w64(unsure) != 0) {
+          asm volatile("" ::: "memory");
+          if (unsure) bin = (int)(t / range);
+        }
+      }
       if (bin == nbins) bin -= 1;
       __hip_atomic_fetch_add(bins + bin, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
     }
@@ -682,19 +697,20 @@ struct HistcBody {
     sb.sync();
     const float lo = a.minvalue, hi = a.maxvalue, range = hi - lo, fn = (float)nbins;
     const float inv_range = 1.0f / range;
+    const float inv_lo = inv_range * (1.0f - 0x1p-21f), inv_hi = inv_range * (1.0f + 0x1p-21f);
     const float *b = a.b.data;
     const int64_t total = a.total_elements;
     auto count4 = [&](const f32x4 v) {
-      count<POW2>(bins, v.x, lo, hi, fn, range, inv_range, nbins);
-      count<POW2>(bins, v.y, lo, hi, fn, range, inv_range, nbins);
-      count<POW2>(bins, v.z, lo, hi, fn, range, inv_range, nbins);
-      count<POW2>(bins, v.w, lo, hi, fn, range, inv_range, nbins);
+      count<POW2>(bins, v.x, lo, hi, fn, range, inv_range, inv_lo, inv_hi, nbins);
+      count<POW2>(bins, v.y, lo, hi, fn, range, inv_range, inv_lo, inv_hi, nbins);
+      count<POW2>(bins, v.z, lo, hi, fn, range, inv_range, inv_lo, inv_hi, nbins);
+      count<POW2>(bins, v.w, lo, hi, fn, range, inv_range, inv_lo, inv_hi, nbins);
     };
     if (hint & HINT_HIST_VEC4) {
       // `head` elements (0..3) precede the first 16-byte boundary; block 0 counts them and the
       // tail with scalar loads, everyone streams the aligned middle.
       const int64_t head = min((int64_t)((hint >> HINT_HIST_HEAD_SHIFT) & 3u), total);
-      if (sb.bid == 0 && (int64_t)sb.tid < head) count<POW2>(bins, b[sb.tid], lo, hi, fn, range, inv_range, nbins);
+      if (sb.bid == 0 && (int64_t)sb.tid < head) count<POW2>(bins, b[sb.tid], lo, hi, fn, range, inv_range, inv_lo, inv_hi, nbins);
       b += head;
       const int64_t rest = total - head;
       const int64_t n4 = rest >> 2;
@@ -714,12 +730,12 @@ struct HistcBody {
       for (; i < n4; i += stride) count4(ld4(b + i * 4));
       if (sb.bid == 0)
         for (int64_t k = (n4 << 2) + sb.tid; k < rest; k += sb.nthreads)
-          count<POW2>(bins, b[k], lo, hi, fn, range, inv_range, nbins);
+          count<POW2>(bins, b[k], lo, hi, fn, range, inv_range, inv_lo, inv_hi, nbins);
     } else {
       const int64_t stride = (int64_t)sb.gstride();
       const int64_t bs = a.b.strides[0];
       for (int64_t i = (int64_t)sb.gtid(); i < total; i += stride)
-        count<POW2>(bins, b[i * bs], lo, hi, fn, range, inv_range, nbins);
+        count<POW2>(bins, b[i * bs], lo, hi, fn, range, inv_range, inv_lo, inv_hi, nbins);
     }
     sb.sync();
     const int64_t as = a.a.strides[0];
