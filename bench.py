@@ -388,7 +388,7 @@ def main():
     h = headline or {}
     n_fast = sum(1 for r in report.values() if r.get("speedup_pct", -1e9) >= 10.0)
     line = {
-        "metric": "fused-pair time vs back-to-back launches (speedup %)",
+        "metric": "fused-pair time vs back-to-back launches (speedup %); GB/s or MH/s vs roofline",
         "value": h.get("speedup_pct"),
         "unit": "%",
         "n_gpus": 1,
