@@ -435,3 +435,61 @@ def test_deep_nesting_is_refused_not_followed():
     with pytest.raises(hfuse_amd.HfuseError) as e:
         Config(seqs, KERNELS_MAP)
     assert e.value.code == L.HF_EPARSE
+
+
+def test_partition_matches_oracle_on_random_kernel_tables():
+    """Seeded random tables (block shapes, Reg, ExecTime), every preset, every split of the
+    enumeration plus the ExecTime split: the library's partition, block shapes, launch threads,
+    launch-bounds hint and index remap equal the oracle's Context wherever the library accepts
+    the variant, and what it refuses is a part that is empty or not a multiple of 64 / BlockDim.Y."""
+    import random
+    rng = random.Random(20240607)
+    checked = refused = 0
+    for case in range(300):
+        rows = []
+        for _ in range(2):
+            y = rng.choice([1, 1, 1, 2, 4, 8, 16])
+            x = rng.choice([32, 64, 128, 192, 256, 320, 512, 768, 1024]) // y
+            if x == 0 or x * y > 1024:
+                x, y = 64, 1
+            rows.append(((x, y, 1), rng.choice([8, 16, 24, 32, 49, 64, 128, 255]), rng.choice([-1.0, 1.0, 17.0, 52.5, 95.0])))
+        total = sum(r[0][0] * r[0][1] for r in rows)
+        if total > 1024:
+            continue
+        names = ("im2col_kernel", "MaxPoolForward")   # any two built kernels: only the table's numbers matter here
+        table = "".join(f"k{i}:\n  KernelName: {names[i]}\n  HasBarriers: false\n  BlockDim:\n    X: {r[0][0]}\n    Y: {r[0][1]}\n    Z: 1\n"
+                        f"  Reg: {r[1]}\n" + (f"  ExecTime: {r[2]}\n" if r[2] > 0 else "") for i, r in enumerate(rows))
+        cfg = Config("- File: f\n  Kernels:\n    - k0\n    - k1\n", table)
+        assert cfg.num_splits(0) == len(O.enumerate_splits(rows, granule=64))
+        variants = [(idx, [(rows[0][0], rows[0][1], float(128 * (idx + 1))), (rows[1][0], rows[1][1], float(total - 128 * (idx + 1)))])
+                    for idx in range(cfg.num_splits(0))]
+        if rows[0][2] > 0 and rows[1][2] > 0:
+            variants.append((L.HF_SPLIT_EXECTIME, rows))
+        for idx, ex in variants:
+            for preset, lb in (("hfuse", False), ("hfuse_lb", True)):
+                try:
+                    want = O.context(ex, launch_bound=lb, imbalanced=True, granule=64, reg_file=4 * 512 * 64, max_threads=2048)
+                except ValueError:
+                    want = None
+                try:
+                    got = cfg.plan(0, preset, idx).partition
+                except hfuse_amd.HfuseError as e:
+                    assert e.code == L.HF_EINVAL
+                    refused += 1
+                    if want is not None:   # the reference's arithmetic allows it; here a part must be whole wavefronts / rows
+                        parts = [want.hi[h] - want.lo[h] for h in range(2)]
+                        assert any(p == 0 or p % 64 or p % rows[h][0][1] for h, p in enumerate(parts)), (rows, idx, parts)
+                    continue
+                assert want is not None, (rows, idx)
+                assert list(got.lo) == list(want.lo) and list(got.hi) == list(want.hi), (rows, idx)
+                for h in range(2):
+                    assert (got.block_dim[h].x, got.block_dim[h].y) == (want.block_dim[h].x, want.block_dim[h].y)
+                assert got.launch_threads == want.launch_threads and got.launch_blocks == want.launch_blocks
+                checked += 1
+        for preset, lb in (("vfuse", False), ("vfuse_lb", True)):
+            want = O.context(rows, base_line=True, launch_bound=lb, imbalanced=False, granule=64, reg_file=4 * 512 * 64, max_threads=2048)
+            got = cfg.plan(0, preset, 0).partition
+            assert list(got.lo) == [0, 0] == list(want.lo) and list(got.hi) == list(want.hi)
+            assert got.launch_threads == want.launch_threads and got.launch_blocks == want.launch_blocks
+            checked += 1
+    assert checked > 800 and refused > 10
