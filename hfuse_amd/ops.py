@@ -144,7 +144,7 @@ def histc(x, bins: int = 100, min: float = 0.0, max: float = 0.0) -> Op:
 
 @dataclass
 class SearchOp(Op):
-    grid: int = 0          # ethash only: the launch grid fixes the nonce count (grid * 128)
+    count: int = 0         # ethash only: nonces to scan; the launch grid is derived from it
 
 
 def sha256d_search(header: bytes, target64: int, start: int, count: int) -> SearchOp:
@@ -170,11 +170,12 @@ def blake2b_search(header: bytes, target64: int, start: int, count: int) -> Sear
 
 
 def ethash_search(dag, dag_items: int, header: bytes, target64: int, start: int, count: int) -> SearchOp:
-    """Ethash hashimoto over a resident DAG of `dag_items` 128-byte items; `count` is rounded up
-    to a multiple of 128 (the original's grid * block nonces)."""
+    """Ethash hashimoto over a resident DAG of `dag_items` 128-byte items.  The kernel scans
+    grid * block nonces like the original, so `count` is rounded up to a multiple of its block
+    (128 threads natively, its share of the fused block in a fused launch)."""
     H.ethash_set_constants(dag, dag_items, header, target64)
     res = H.new_search_results()
-    return SearchOp("ethash_search", H.ethash_args(res, start), (res,), (res, dag), grid=(int(count) + 127) // 128)
+    return SearchOp("ethash_search", H.ethash_args(res, start), (res,), (res, dag), count=int(count))
 
 
 def hits(op: SearchOp):
@@ -199,7 +200,11 @@ def _config(cfg: Optional[H.Config]) -> H.Config:
 
 def run(op: Op, stream=None):
     """Launch one original kernel; returns its outputs (a tuple)."""
-    H.launch_native(op.kernel, op.args, getattr(op, "grid", 0), 0, stream=stream)
+    count = getattr(op, "count", 0)
+    if count:   # ethash: grid * 128 threads cover the requested nonces
+        H.launch_native(op.kernel, op.args, (count + 127) // 128, 128, stream=stream)
+    else:
+        H.launch_native(op.kernel, op.args, stream=stream)
     return op.outputs
 
 
@@ -209,12 +214,19 @@ def run_fused(op1: Op, op2: Op, cfg: Optional[H.Config] = None, preset: str = "h
     The pair is looked up in the fusion list of `cfg` (default: the shipped list) in either
     order; a pair the list does not name raises KeyError."""
     c = _config(cfg)
-    grid = max(getattr(op1, "grid", 0), getattr(op2, "grid", 0))     # ethash's exact grid, 0 otherwise
     try:
         first, second = op1, op2
         index = c.find_fusion(op1.kernel, op2.kernel)
     except KeyError:
         first, second = op2, op1
         index = c.find_fusion(op2.kernel, op1.kernel)
-    c.plan(index, preset).launch(first.args, second.args, grid_blocks=grid, stream=stream)
+    plan = c.plan(index, preset)
+    grid = 0
+    part = plan.partition
+    for half, op in enumerate((first, second)):   # ethash: the grid times its share of the block covers the nonces
+        count = getattr(op, "count", 0)
+        if count:
+            threads = part.hi[half] - part.lo[half]
+            grid = max(grid, (count + threads - 1) // threads)
+    plan.launch(first.args, second.args, grid_blocks=grid, stream=stream)
     return op1.outputs, op2.outputs

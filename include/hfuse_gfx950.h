@@ -293,7 +293,13 @@ typedef struct {
   hf_search_hit hit[HF_MAX_SEARCH_RESULTS]; /* unordered; callers sort by nonce                  */
 } hf_search_results;
 
-/* ethash_search(volatile Search_results*, uint64_t) -- scripts/data/ethminer_event.csv:9 */
+/*
+ * ethash_search(volatile Search_results*, uint64_t) -- scripts/data/ethminer_event.csv:9.
+ * Like the original (gid = blockIdx * blockDim + threadIdx) it takes no count: a launch scans
+ * grid_blocks * block threads nonces from start_nonce, where the block is the kernel's own in
+ * a native launch and its share of the fused block (hf_plan_partition: hi[k] - lo[k]) in a
+ * fused one.  grid_blocks <= 0 means 8192 blocks, the reference traces' launch.
+ */
 typedef struct {
   hf_search_results *g_output;
   uint64_t start_nonce;

@@ -244,3 +244,73 @@ def test_zero_nonces_find_nothing(cuda, cfg):
     want = oracle_hits(O.sha256d_search(hdr, 0, 1 << 14, EASY12))
     assert want[0] > 0 and H.read_search_results(r1) == want
     assert H.read_search_results(r2)[0] == 0
+
+
+def test_random_fused_search_configurations(cuda, cfg):
+    """Seeded random walk over the seven search pairs: random nonce windows (wrapping 2^32 too),
+    fused block shapes up to 512 threads, lending, partition mode, caller grids.  The fused found
+    sets must equal the oracle's for the same windows."""
+    import random
+    from hfuse_amd import _lib as L
+    rng = random.Random(0xE7A5)
+    n_items = 4099                      # not a power of two: the modulo path
+    dag = _dag(cuda, n_items, SEED)
+    header = O.seeded_bytes(32, SEED + 20)
+    hs, hb, hc = (O.seeded_bytes(80, SEED + 21 + k) for k in range(3))
+    eth_target = (1 << 55) - 1          # about one hit in 500 nonces: stays below the 64 records kept
+    H.ethash_set_constants(dag, n_items, header, eth_target)
+    H.sha256d_set_block(hs, EASY10)
+    H.sia_blake2b_set_block(hb)
+    H.blake2b_set_block(hc)
+    names = ("ethash_search", "sha256d_gpu_hash_shared", "sia_blake2b_gpu_hash", "blake2b_gpu_hash")
+    pairs = [(i, k1, k2) for i, (_, k1, k2) in enumerate(cfg.fusions()) if k1 in names and k2 in names]
+    assert len(pairs) == 7
+
+    def expected(k, start, count):
+        if k == "ethash_search":
+            return oracle_hits(O.ethash_search(None, SEED, n_items, header, start, count, eth_target))
+        if k == "sha256d_gpu_hash_shared":
+            return oracle_hits(O.sha256d_search(hs, start, count, EASY10))
+        if k == "sia_blake2b_gpu_hash":
+            return oracle_hits(O.sia_search(hb, start, count, EASY10))
+        want = []                        # ccminer layout: brute force with the oracle's single-nonce digest
+        for t in range(count):
+            nonce = (start + t) & 0xFFFFFFFF
+            d = O.ccminer_blake2b_80(hc, nonce)
+            if int.from_bytes(d[:8], "big") <= EASY10:
+                want.append((nonce, d, bytes(32)))
+        return len(want), sorted(want)
+
+    for case in range(24):
+        i, k1, k2 = rng.choice(pairs)
+        grid = rng.choice([8, 24, 33]) if "ethash_search" in (k1, k2) else rng.choice([0, 0, 5, 19])
+        starts = [rng.choice([0, 12345, 0xFFFFFF00, rng.randrange(1 << 32)]) for _ in range(2)]
+        plan = cfg.plan(i, rng.choice(["hfuse", "hfuse_lb", "vfuse"]))
+        threads = [128, 128]             # the kernel table's blocks; a vertical plan keeps them
+        if "vfuse" not in plan.name:
+            t1 = 64 * rng.randint(1, 7)
+            t2 = 64 * rng.randint(1, 8 - t1 // 64)
+            plan.set_block(t1, t2)
+            plan.set_lending(rng.random() < 0.5)
+            if rng.random() < 0.3:
+                plan.set_barrier_mode(L.HF_BARRIER_BLOCKIDX)
+            threads = [t1, t2]
+        # Ethash scans gridDim * blockDim nonces like the original: its share of the fused block counts
+        counts = [grid * threads[h] if k == "ethash_search" else rng.choice([1, 1000, 4096, 10007]) for h, k in enumerate((k1, k2))]
+        res, args = [], []
+        for k, st, cnt in zip((k1, k2), starts, counts):
+            r = H.new_search_results()
+            res.append(r)
+            if k == "ethash_search":
+                args.append(H.ethash_args(r, st))
+            elif k == "sha256d_gpu_hash_shared":
+                args.append(H.sha256d_args(r, cnt, st))
+            else:
+                args.append(H.blake2b_args(r, cnt, st, EASY10))
+        label = f"case {case}: {k1}[{starts[0]:#x}+{counts[0]}] + {k2}[{starts[1]:#x}+{counts[1]}] grid {grid} block {threads}"
+        plan.launch(args[0], args[1], grid_blocks=grid)
+        sync()
+        for k, r, st, cnt in zip((k1, k2), res, starts, counts):
+            if k == "ethash_search" and st + cnt > (1 << 32):
+                continue   # 64-bit nonces do not wrap; the 32-bit window helpers above do
+            assert H.read_search_results(r) == expected(k, st, cnt), f"{label}: {k}"

@@ -692,3 +692,94 @@ def test_two_host_threads_on_their_own_streams(cuda, cfg):
     sync()
     for u in up:
         u.check()
+
+
+def test_random_fused_configurations(cuda, cfg):
+    """Seeded random walk over the tensor pairs of the shipped list: random small shapes (fast and
+    general paths), fused block shapes, lending on / off, every partition mode legal for the pair,
+    per-half grids; every launch is checked against the oracle / PyTorch CPU like the native kernels."""
+    import random
+    rng = random.Random(0xF05E)
+
+    def rand_im2col():
+        k = rng.choice([(3, 3), (3, 3), (1, 1), (2, 3), (5, 5)])
+        p = (1, 1) if k == (3, 3) and rng.random() < 0.7 else (rng.randint(0, k[0] // 2), rng.randint(0, k[1] // 2))
+        s = (1, 1) if rng.random() < 0.7 else (rng.randint(1, 2), rng.randint(1, 2))
+        h, w = rng.randint(5, 14), rng.choice([8, 12, 16, 7, 9, 13])
+        return Im2col(cuda, rng.randint(1, 3), rng.randint(1, 5), h, w, k, p, s, (1, 1), seed=rng.randint(0, 999))
+
+    def rand_pool():
+        k, s, p = rng.choice([((3, 3), (2, 2), (1, 1)), ((2, 2), (2, 2), (0, 0)), ((3, 2), (1, 2), (1, 0)), ((2, 2), (1, 1), (1, 1))])
+        h, w = rng.choice([8, 12, 16, 9, 11]), rng.choice([8, 16, 24, 10, 13])
+        return MaxPool(cuda, rng.randint(1, 3), rng.randint(1, 4), h, w, k, s, p, seed=rng.randint(0, 999))
+
+    class BnStatsSmall(BnStats):
+        """Planes of a few elements can have a mean next to zero, where an element-wise relative error
+        says nothing; the mean is held to 1e-5 of the plane's scale max(|mean|, std) instead."""
+
+        def check(self):
+            n, c = self.x.shape[:2]
+            m64, i64 = O.bn_stats_f64(self.x.reshape(n, c, -1).numpy(), 1e-5)
+            gm, gi = self.mean.cpu().numpy().astype(np.float64), self.inv.cpu().numpy()
+            assert np.max(np.abs(gm - m64) / np.maximum(np.abs(m64), 1.0 / i64)) < BN_TOL
+            assert rel_err(gi, i64) < BN_TOL, rel_err(gi, i64)
+            self.mean.fill_(float("nan"))
+            self.inv.fill_(float("nan"))
+
+    def rand_bn():
+        return BnStatsSmall(cuda, rng.randint(1, 5), rng.randint(1, 12), rng.randint(1, 7), rng.choice([1, 3, 4, 8]), seed=rng.randint(0, 999))
+
+    def rand_up():
+        h, w = rng.randint(1, 9), rng.choice([2, 4, 6, 8, 5, 7])
+        out = (2 * h, 2 * w) if rng.random() < 0.6 else (rng.randint(1, 20), rng.randint(1, 20))
+        return Upsample(cuda, rng.randint(1, 3), rng.randint(1, 4), h, w, out, seed=rng.randint(0, 999))
+
+    def rand_bilinear():
+        h, w = rng.randint(1, 9), rng.choice([2, 4, 6, 8, 5, 7])
+        out = (2 * h, 2 * w) if rng.random() < 0.5 else (rng.randint(1, 20), rng.choice([4, 8, 12, 5, 9]))
+        return Bilinear(cuda, rng.randint(1, 3), rng.randint(1, 4), h, w, out, align=rng.random() < 0.5, seed=rng.randint(0, 999))
+
+    def rand_hist():
+        nbins, lo, hi = rng.choice([(1024, 0.0, 1.0), (16, 0.0, 1.0), (100, -1.0, 2.0), (7, 0.0, 3.0)])
+        return Histc(cuda, rng.choice([1, 63, 1000, 40001]), nbins, lo, hi, seed=rng.randint(0, 999))
+
+    makers = {"im2col_kernel": rand_im2col, "MaxPoolForward": rand_pool, "batch_norm_collect_statistics_kernel": rand_bn,
+              "upsample_nearest2d_out_frame": rand_up, "upsample_bilinear2d_out_frame": rand_bilinear, "kernelHistogram1D": rand_hist}
+    sync_kernels = {"batch_norm_collect_statistics_kernel", "kernelHistogram1D"}
+    pairs = [(i, k1, k2) for i, (_, k1, k2) in enumerate(cfg.fusions()) if k1 in makers and k2 in makers]
+    assert len(pairs) == 15
+    launched = 0
+    for case in range(120):
+        i, k1, k2 = rng.choice(pairs)
+        a, b = makers[k1](), makers[k2]()
+        plan = cfg.plan(i, rng.choice(["hfuse", "hfuse", "hfuse_lb", "vfuse"]))
+        label = f"case {case}: {k1} + {k2}"
+        if not plan.name.count("vfuse"):
+            y1 = cfg.kernel(k1).block_dim.y
+            y2 = cfg.kernel(k2).block_dim.y
+            t1 = 64 * rng.randint(1, 8)
+            t2 = 64 * rng.randint(1, (1024 - t1) // 64)
+            if t1 % y1 == 0 and t2 % y2 == 0 and rng.random() < 0.8:
+                plan.set_block(t1, t2)
+                label += f" block {t1}+{t2}"
+            plan.set_lending(rng.random() < 0.5)
+            modes = [None, L.HF_BARRIER_BLOCKIDX]
+            if k1 in sync_kernels and k2 in sync_kernels:
+                modes.append(L.HF_BARRIER_MATCHED)
+            mode = rng.choice(modes)
+            if mode is not None:
+                plan.set_barrier_mode(mode)
+                label += f" mode {mode}"
+            if rng.random() < 0.3:
+                g = (rng.randint(1, 40), rng.randint(1, 40))
+                plan.set_grids(*g)
+                label += f" grids {g}"
+        plan.launch(a.args, b.args, grid_blocks=rng.choice([0, 0, 0, 3, 17]))
+        sync()
+        try:
+            a.check()
+            b.check()
+        except AssertionError as e:
+            raise AssertionError(f"{label}: {e}") from e
+        launched += 1
+    assert launched == 120
