@@ -166,13 +166,22 @@ def run_search_pair(cfg, name, log2_a, log2_b, sweep, fused_only, iters=2):
         res["t_a_ms"] = base.time(0, [a1], [a2], 1, iters, grid) / iters
         res["t_b_ms"] = base.time(1, [a1], [a2], 1, iters, 0) / iters
         res["t_b2b_ms"] = base.time(2, [a1], [a2], 0, iters, grid) / iters
+    def grid_of(plan):
+        # ethash scans grid * (its share of the fused block) nonces: keep the range at `na`
+        if not ethash:
+            return grid
+        share = plan.partition.hi[0] - plan.partition.lo[0]
+        assert na % share == 0
+        return na // share
+
     best = None
     for label, plan in plans:
-        t = plan.time(3, [a1], [a2], 0, 1, grid)
+        t = plan.time(3, [a1], [a2], 0, 1, grid_of(plan))
         if best is None or t < best[0]:
             best = (t, label, plan)
     _, label, plan = best
-    res["t_fused_ms"] = plan.time(3, [a1], [a2], 0, iters, grid) / iters
+    fused_grid = grid_of(plan)
+    res["t_fused_ms"] = plan.time(3, [a1], [a2], 0, iters, fused_grid) / iters
     if not fused_only:
         res["t_vfuse_ms"] = cfg.plan(cfg.find_fusion(k1, k2), "vfuse").time(3, [a1], [a2], 0, 1, grid)
         res["t_two_streams_ms"] = base.time(4, [a1], [a2], 0, 1, grid)
@@ -183,7 +192,7 @@ def run_search_pair(cfg, name, log2_a, log2_b, sweep, fused_only, iters=2):
     # Correctness of what was just timed: one more fused pass into fresh buffers, every hit
     # re-hashed by the oracle, and the found sets compared with the native kernels' found sets.
     fa, fb, f1, f2 = fresh()
-    plan.launch(f1, f2, grid_blocks=grid)
+    plan.launch(f1, f2, grid_blocks=fused_grid)
     na_, nb_, n1, n2 = fresh()
     H.launch_native(k1, n1, grid, 128)
     H.launch_native(k2, n2, 0, 128)

@@ -110,13 +110,18 @@ def tune(cfg: H.Config, fusion_index: int, args1: Sequence, args2: Sequence, *,
          blocks: Optional[Sequence[Tuple[int, int]]] = None, lending: Sequence[bool] = (True, False),
          barrier_modes: Sequence[Optional[int]] = (None,), grids: Sequence[Tuple[int, int]] = ((0, 0),),
          probe_iters: int = 20, final_iters: int = 100, finalists: int = 4, warmup: int = 3,
-         grid_blocks: int = 0, verbose: bool = False) -> TuneResult:
+         grid_blocks=0, verbose: bool = False) -> TuneResult:
     """Sweep the candidates of one pair on the caller's argument sets and return the fastest.
 
     args1[i] / args2[i] are argument structs of independent buffer sets the timed launches rotate
     through (hf_time_pair).  Every candidate gets `probe_iters` launches; the `finalists` fastest
     are timed again over `final_iters` launches in three interleaved rounds, together with the
-    back-to-back native launches and the untuned table split, and the median decides."""
+    back-to-back native launches and the untuned table split, and the median decides.
+
+    `grid_blocks` is the launch grid (0: the library's) or a function (threads1, threads2) -> grid
+    for kernels whose grid fixes their work: Ethash scans grid * its-threads nonces, so a fair
+    sweep gives every block shape the grid that covers the same nonce range."""
+    grid_of = grid_blocks if callable(grid_blocks) else (lambda t1, t2: grid_blocks)
     file, k1, k2 = cfg.fusion(fusion_index)
     if blocks is None:
         blocks = block_candidates(cfg, fusion_index, step=2 * WAVE)
@@ -128,7 +133,7 @@ def tune(cfg: H.Config, fusion_index: int, args1: Sequence, args2: Sequence, *,
             plan = _make_plan(cfg, fusion_index, c)
         except H.HfuseError:
             continue   # not legal for this pair (BlockDim.Y, barrier mode, block cap)
-        t = plan.time(3, args1, args2, warmup, probe_iters, grid_blocks) / probe_iters
+        t = plan.time(3, args1, args2, warmup, probe_iters, grid_of(c.threads1, c.threads2)) / probe_iters
         probed.append((t, c, plan))
         if verbose:
             print(f"  {c.label():28s} {t * 1e3:9.2f} us", file=sys.stderr, flush=True)
@@ -140,8 +145,9 @@ def tune(cfg: H.Config, fusion_index: int, args1: Sequence, args2: Sequence, *,
     base_cfg_plan = cfg.plan(fusion_index, "hfuse", 0)
     d1 = cfg.kernel(k1).block_dim
     d2 = cfg.kernel(k2).block_dim
+    base1, base2 = d1.x * d1.y * d1.z, d2.x * d2.y * d2.z
     try:
-        base_cfg_plan.set_block(d1.x * d1.y * d1.z, d2.x * d2.y * d2.z)
+        base_cfg_plan.set_block(base1, base2)
         base_ok = True
     except H.HfuseError:
         base_ok = False
@@ -149,10 +155,10 @@ def tune(cfg: H.Config, fusion_index: int, args1: Sequence, args2: Sequence, *,
     s_b2b, s_table = [], []
     for _ in range(3):
         for i, (_, _, plan) in enumerate(final):
-            samples[i].append(plan.time(3, args1, args2, 2, final_iters, grid_blocks) / final_iters)
-        s_b2b.append(final[0][2].time(2, args1, args2, 2, final_iters, grid_blocks) / final_iters)
+            samples[i].append(plan.time(3, args1, args2, 2, final_iters, grid_of(final[i][1].threads1, final[i][1].threads2)) / final_iters)
+        s_b2b.append(final[0][2].time(2, args1, args2, 2, final_iters, grid_of(base1, base2)) / final_iters)
         if base_ok:
-            s_table.append(base_cfg_plan.time(3, args1, args2, 2, final_iters, grid_blocks) / final_iters)
+            s_table.append(base_cfg_plan.time(3, args1, args2, 2, final_iters, grid_of(base1, base2)) / final_iters)
     med = sorted(((statistics.median(v), i) for i, v in samples.items()))
     # Timings this close are the same speed: among them prefer the library's defaults
     # (lending on, the pair's own barrier design) so that noise does not write keys.
@@ -262,8 +268,11 @@ def main(argv=None) -> int:
         else:
             sp = W.SearchPair(k1, k2, args.search_log2, args.search_log2)
             _, _, a1, a2 = sp.fresh()
+            # ethash scans grid * its-threads nonces: every block shape gets the grid for the same range
+            eth = 0 if k1 == "ethash_search" else 1 if k2 == "ethash_search" else None
+            grid = (lambda t1, t2: sp.nonces[eth] // (t1, t2)[eth]) if eth is not None else 0
             r = tune(cfg, i, [a1], [a2], blocks=blocks, lending=(True,), probe_iters=1, final_iters=2,
-                     warmup=0, grid_blocks=sp.grid, verbose=args.verbose)
+                     warmup=0, grid_blocks=grid, verbose=args.verbose)
             del sp
         torch.cuda.empty_cache()
         gain = (r.t_table_ms / r.t_best_ms - 1.0) * 100.0 if r.t_table_ms == r.t_table_ms else float("inf")

@@ -143,7 +143,8 @@ class SearchPair:
     """Two nonce searches with their constants uploaded: `fresh()` -> (results1, results2, args1, args2).
 
     Constants are per process (hf_*_set_block), so only one SearchPair is live at a time.
-    `grid` is the exact grid Ethash needs (its nonce count is gridDim * 128); 0 for the others."""
+    `grid` is the grid a native Ethash launch of 128-thread blocks needs for its nonce count (Ethash
+    scans gridDim * blockDim nonces); a fused launch divides by Ethash's share of the block instead."""
 
     ETHASH_ITEMS = 1 << 25            # 4 GiB of 128-byte DAG items
     ETHASH_TARGET = (1 << 40) - 1     # 24 leading zero bits
