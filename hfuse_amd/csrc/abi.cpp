@@ -351,7 +351,7 @@ int prepare_histc(const hf_histc_args &a, Prepared &p) {
   if (a.a.sizes[0] != a.nbins) return fail(HF_EINVAL, "kernelHistogram1D: output length is not nbins");
   if (a.b.sizes[0] != a.total_elements) return fail(HF_EINVAL, "kernelHistogram1D: totalElements is not the input length");
   if (a.a.strides[0] != 1) return fail(HF_EUNSUPPORTED, "kernelHistogram1D: output must be contiguous");
-  if (a.nbins > 15360) return fail(HF_EUNSUPPORTED, "kernelHistogram1D: more bins than fit the LDS budget (15360)");
+  const bool global_bins = a.nbins > 15360;  // beyond the LDS budget the bins are counted in global memory
   int64_t far;
   if (a.b.strides[0] < 0 || !product(far, {a.total_elements > 0 ? a.total_elements - 1 : 0, a.b.strides[0]}))
     return fail(HF_EINVAL, "kernelHistogram1D: negative or oversized input stride");
@@ -364,8 +364,9 @@ int prepare_histc(const hf_histc_args &a, Prepared &p) {
   int exp2 = 0;
   const float range = a.maxvalue - a.minvalue;
   const bool pow2 = std::frexp(range, &exp2) == 0.5f && exp2 > -100 && exp2 < 100;
-  p.hint = (fast ? HINT_HIST_VEC4 : HINT_GENERIC) | (pow2 ? HINT_HIST_POW2 : 0) | (head << HINT_HIST_HEAD_SHIFT);
-  p.lds = (unsigned)a.nbins * 4u;
+  p.hint = (fast ? HINT_HIST_VEC4 : HINT_GENERIC) | (pow2 ? HINT_HIST_POW2 : 0) | (head << HINT_HIST_HEAD_SHIFT) |
+           (global_bins ? HINT_HIST_GLOBAL : 0);
+  p.lds = global_bins ? 0u : (unsigned)a.nbins * 4u;
   p.items = fast ? (unsigned long long)(a.total_elements + 3) / 4 : (unsigned long long)a.total_elements;
   return HF_OK;
 }

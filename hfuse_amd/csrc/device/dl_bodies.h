@@ -13,7 +13,7 @@
 namespace hfuse {
 
 // Hints (0 always means the general path).
-enum { HINT_GENERIC = 0, HINT_IM2COL_3X3_S1P1 = 1, HINT_POOL_K3S2P1 = 1, HINT_POOL_K2S2P0 = 2, HINT_UP_2X = 1, HINT_BN_VEC4 = 1, HINT_HIST_VEC4 = 1, HINT_HIST_POW2 = 2, HINT_HIST_HEAD_SHIFT = 4 /* bits 4-5: elements before the first 16-byte boundary */, HINT_BILINEAR_VEC4 = 1, HINT_BILINEAR_2X = 2,
+enum { HINT_GENERIC = 0, HINT_IM2COL_3X3_S1P1 = 1, HINT_POOL_K3S2P1 = 1, HINT_POOL_K2S2P0 = 2, HINT_UP_2X = 1, HINT_BN_VEC4 = 1, HINT_HIST_VEC4 = 1, HINT_HIST_POW2 = 2, HINT_HIST_GLOBAL = 8 /* more bins than the LDS budget: count straight into global memory */, HINT_HIST_HEAD_SHIFT = 4 /* bits 4-5: elements before the first 16-byte boundary */, HINT_BILINEAR_VEC4 = 1, HINT_BILINEAR_2X = 2,
        // general path with 32-bit index arithmetic: every tensor of the call has fewer than 2^31 elements
        HINT_IDX32 = 0x100 };
 
@@ -657,7 +657,7 @@ struct HistcBody {
   // bin = (int)((v - min) * nbins / (max - min)) in fp32, bin == nbins -> nbins - 1.
   // POW2: max - min is a power of two, so the correctly rounded division equals the
   // multiplication by its (exact) reciprocal and the IEEE division sequence is not needed.
-  template <bool POW2>
+  template <bool POW2, bool GLOBAL>
   static __device__ __forceinline__ void count(unsigned *bins, float v, float lo, float hi, float scale_n, float range,
                                                float inv_range, float inv_lo, float inv_hi, int nbins) {
     if (v >= lo && v <= hi) {
@@ -679,21 +679,32 @@ struct HistcBody {
         }
       }
       if (bin == nbins) bin -= 1;
-      __hip_atomic_fetch_add(bins + bin, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+      if constexpr (GLOBAL) unsafeAtomicAdd(reinterpret_cast<float *>(bins) + bin, 1.0f);
+      else __hip_atomic_fetch_add(bins + bin, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
     }
   }
 
   template <class SB>
   static __device__ void run(const Args &a, SB &sb, unsigned char *lds, unsigned hint) {
-    if (hint & HINT_HIST_POW2) body<true>(a, sb, lds, hint);
-    else body<false>(a, sb, lds, hint);
+    // The original picks shared or global memory for the bins by what fits; so does the host here.
+    if (hint & HINT_HIST_GLOBAL) {
+      if (hint & HINT_HIST_POW2) body<true, true>(a, sb, lds, hint);
+      else body<false, true>(a, sb, lds, hint);
+    } else if (hint & HINT_HIST_POW2) {
+      body<true, false>(a, sb, lds, hint);
+    } else {
+      body<false, false>(a, sb, lds, hint);
+    }
   }
 
-  template <bool POW2, class SB>
+  // GLOBAL: every element adds 1.0f to its bin of the (contiguous) output directly; the two
+  // synchronisation points stay, so a partner that shares the hardware barrier still matches.
+  template <bool POW2, bool GLOBAL, class SB>
   static __device__ __forceinline__ void body(const Args &a, SB &sb, unsigned char *lds, unsigned hint) {
-    unsigned *bins = reinterpret_cast<unsigned *>(lds);
+    unsigned *bins = GLOBAL ? reinterpret_cast<unsigned *>(a.a.data) : reinterpret_cast<unsigned *>(lds);
     const int nbins = a.nbins;
-    for (int i = (int)sb.tid; i < nbins; i += (int)sb.nthreads) bins[i] = 0;
+    if constexpr (!GLOBAL)
+      for (int i = (int)sb.tid; i < nbins; i += (int)sb.nthreads) bins[i] = 0;
     sb.sync();
     const float lo = a.minvalue, hi = a.maxvalue, range = hi - lo, fn = (float)nbins;
     const float inv_range = 1.0f / range;
@@ -701,16 +712,16 @@ struct HistcBody {
     const float *b = a.b.data;
     const int64_t total = a.total_elements;
     auto count4 = [&](const f32x4 v) {
-      count<POW2>(bins, v.x, lo, hi, fn, range, inv_range, inv_lo, inv_hi, nbins);
-      count<POW2>(bins, v.y, lo, hi, fn, range, inv_range, inv_lo, inv_hi, nbins);
-      count<POW2>(bins, v.z, lo, hi, fn, range, inv_range, inv_lo, inv_hi, nbins);
-      count<POW2>(bins, v.w, lo, hi, fn, range, inv_range, inv_lo, inv_hi, nbins);
+      count<POW2, GLOBAL>(bins, v.x, lo, hi, fn, range, inv_range, inv_lo, inv_hi, nbins);
+      count<POW2, GLOBAL>(bins, v.y, lo, hi, fn, range, inv_range, inv_lo, inv_hi, nbins);
+      count<POW2, GLOBAL>(bins, v.z, lo, hi, fn, range, inv_range, inv_lo, inv_hi, nbins);
+      count<POW2, GLOBAL>(bins, v.w, lo, hi, fn, range, inv_range, inv_lo, inv_hi, nbins);
     };
     if (hint & HINT_HIST_VEC4) {
       // `head` elements (0..3) precede the first 16-byte boundary; block 0 counts them and the
       // tail with scalar loads, everyone streams the aligned middle.
       const int64_t head = min((int64_t)((hint >> HINT_HIST_HEAD_SHIFT) & 3u), total);
-      if (sb.bid == 0 && (int64_t)sb.tid < head) count<POW2>(bins, b[sb.tid], lo, hi, fn, range, inv_range, inv_lo, inv_hi, nbins);
+      if (sb.bid == 0 && (int64_t)sb.tid < head) count<POW2, GLOBAL>(bins, b[sb.tid], lo, hi, fn, range, inv_range, inv_lo, inv_hi, nbins);
       b += head;
       const int64_t rest = total - head;
       const int64_t n4 = rest >> 2;
@@ -730,14 +741,15 @@ struct HistcBody {
       for (; i < n4; i += stride) count4(ld4(b + i * 4));
       if (sb.bid == 0)
         for (int64_t k = (n4 << 2) + sb.tid; k < rest; k += sb.nthreads)
-          count<POW2>(bins, b[k], lo, hi, fn, range, inv_range, inv_lo, inv_hi, nbins);
+          count<POW2, GLOBAL>(bins, b[k], lo, hi, fn, range, inv_range, inv_lo, inv_hi, nbins);
     } else {
       const int64_t stride = (int64_t)sb.gstride();
       const int64_t bs = a.b.strides[0];
       for (int64_t i = (int64_t)sb.gtid(); i < total; i += stride)
-        count<POW2>(bins, b[i * bs], lo, hi, fn, range, inv_range, inv_lo, inv_hi, nbins);
+        count<POW2, GLOBAL>(bins, b[i * bs], lo, hi, fn, range, inv_range, inv_lo, inv_hi, nbins);
     }
     sb.sync();
+    if constexpr (GLOBAL) return;
     const int64_t as = a.a.strides[0];
     for (int i = (int)sb.tid; i < nbins; i += (int)sb.nthreads) {
       const unsigned c = bins[i];

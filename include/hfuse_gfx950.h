@@ -270,7 +270,10 @@ typedef struct {
  * a = output counts (fp32, caller-zeroed, accumulated with atomics),
  * p = partial output (unused in SHARED mode), b = input.  getOp is the
  * constant-1 functor of histc; a NULL function pointer slot keeps the arity.
- * Only contiguous 1-D `a` and `b` are built (HF_EUNSUPPORTED otherwise).
+ * Only 1-D tensors and a contiguous `a` are built (HF_EUNSUPPORTED otherwise).
+ * Up to 15360 bins are counted in LDS and flushed once per workgroup; more bins
+ * are counted in global memory directly, as the original's GLOBAL memory type
+ * (fp32 counts stay exact up to 2^24 per bin).
  */
 typedef struct {
   hf_tensorinfo a, p, b;

@@ -347,6 +347,32 @@ def test_histc_bin_edges_with_any_range(cuda, nbins, lo, hi):
     assert np.array_equal(got, O.histc(x.numpy(), nbins, lo, hi))
 
 
+@pytest.mark.parametrize("nbins,n", [(15361, 200000), (100000, 300000), (1 << 20, 50000)])
+def test_histc_more_bins_than_lds_holds(cuda, nbins, n):
+    """Beyond 15360 bins the counts go straight to global memory (the original also switches from
+    shared to global memory by what fits); alone and fused with batch norm in every partition mode."""
+    t = Histc(cuda, n, nbins, 0.0, 1.0)
+    H.launch_native("kernelHistogram1D", t.args)
+    sync()
+    t.check()
+    cfg = hfuse_amd_default()
+    i = cfg.find_fusion("kernelHistogram1D", "batch_norm_collect_statistics_kernel")
+    for mode in (None, L.HF_BARRIER_MATCHED, L.HF_BARRIER_BLOCKIDX):
+        plan = cfg.plan(i)
+        if mode is not None:
+            plan.set_barrier_mode(mode)
+        bn = BnStats(cuda, 4, 9, 6, 6)
+        plan.launch(t.args, bn.args)
+        sync()
+        t.check()
+        bn.check()
+
+
+def hfuse_amd_default():
+    import hfuse_amd
+    return hfuse_amd.default_config()
+
+
 def test_histc_out_of_range_and_accumulation(cuda):
     x = torch.tensor([-0.5, 0.0, 0.999, 1.0, 1.5, float("nan"), 0.3, 0.3])
     t = Histc(cuda, 8, 4, 0.0, 1.0, x=x)
