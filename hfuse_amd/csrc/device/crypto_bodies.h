@@ -98,7 +98,7 @@ struct Sha256dBody {
   static constexpr bool kFlat = true;
 
   template <class SB>
-  static __device__ void run(const Args &a, SB &sb, unsigned char *, unsigned) {
+  static __device__ __forceinline__ void run(const Args &a, SB &sb, unsigned char *, unsigned) {
     const u32 stride = sb.gstride();
     for (u32 t = sb.gtid(); t < a.threads; t += stride) {
       const u32 nonce = a.start_nonce + t;
@@ -224,7 +224,7 @@ struct Blake2bBody {
   static constexpr bool kFlat = true;
 
   template <class SB>
-  static __device__ void run(const Args &a, SB &sb, unsigned char *, unsigned) {
+  static __device__ __forceinline__ void run(const Args &a, SB &sb, unsigned char *, unsigned) {
     const u32 stride = sb.gstride();
     for (u32 t = sb.gtid(); t < a.threads; t += stride) {
       const u32 nonce = a.start_nonce + t;
@@ -319,7 +319,7 @@ struct EthashBody {
   static constexpr int kGroup = 8, kParallel = 4, kAccesses = 64;
 
   template <class SB>
-  static __device__ void run(const Args &a, SB &sb, unsigned char *, unsigned) {
+  static __device__ __forceinline__ void run(const Args &a, SB &sb, unsigned char *, unsigned) {
     const u32 gid = sb.bid * sb.nthreads + sb.tid;
     const u64 nonce = a.start_nonce + gid;
     const int lane_in_group = (int)(sb.tid & (kGroup - 1));

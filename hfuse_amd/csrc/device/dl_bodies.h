@@ -47,7 +47,7 @@ struct Im2colBody {
   static constexpr bool kFlat = true;  // walks one flat index range: may borrow a partner's idle waves
 
   template <class SB>
-  static __device__ void run(const Args &a, SB &sb, unsigned char *, unsigned hint) {
+  static __device__ __forceinline__ void run(const Args &a, SB &sb, unsigned char *, unsigned hint) {
     if (hint == HINT_IM2COL_3X3_S1P1) {
       vec4_3x3(a, sb);
       return;
@@ -150,7 +150,7 @@ struct MaxPoolBody {
   static constexpr bool kFlat = true;
 
   template <class SB>
-  static __device__ void run(const Args &a, SB &sb, unsigned char *, unsigned hint) {
+  static __device__ __forceinline__ void run(const Args &a, SB &sb, unsigned char *, unsigned hint) {
     if (hint == HINT_POOL_K3S2P1) { vec2_s2<3, 1>(a, sb); return; }
     if (hint == HINT_POOL_K2S2P0) { vec2_s2<2, 0>(a, sb); return; }
     if (hint == HINT_IDX32) general<unsigned>(a, sb);
@@ -281,7 +281,7 @@ struct UpsampleNearestBody {
   static constexpr bool kFlat = true;
 
   template <class SB>
-  static __device__ void run(const Args &a, SB &sb, unsigned char *, unsigned hint) {
+  static __device__ __forceinline__ void run(const Args &a, SB &sb, unsigned char *, unsigned hint) {
     if (hint == HINT_UP_2X) {
       // Exact 2x: a lane loads two neighbouring input pixels (8 B) and stores the four
       // output pixels they expand to (16 B) into both output rows, so each load and each
@@ -449,7 +449,7 @@ struct UpsampleBilinearBody {
   }
 
   template <class SB>
-  static __device__ void run(const Args &a, SB &sb, unsigned char *, unsigned hint) {
+  static __device__ __forceinline__ void run(const Args &a, SB &sb, unsigned char *, unsigned hint) {
     const int H1 = (int)a.idata.sizes[2], W1 = (int)a.idata.sizes[3];
     const int H2 = (int)a.odata.sizes[2], W2 = (int)a.odata.sizes[3];
     const unsigned NC = (unsigned)(a.idata.sizes[0] * a.idata.sizes[1]);
@@ -576,7 +576,7 @@ struct BnStatsBody {
   static constexpr unsigned kLdsBytes = 16 * sizeof(Welford) + 16;
 
   template <class SB>
-  static __device__ void run(const Args &a, SB &sb, unsigned char *lds, unsigned hint) {
+  static __device__ __forceinline__ void run(const Args &a, SB &sb, unsigned char *lds, unsigned hint) {
     Welford *part = reinterpret_cast<Welford *>(lds);
     const int N = a.input.sizes[0], C = a.input.sizes[1], L = a.input.sizes[2];
     for (int plane = (int)sb.bid; plane < C; plane += (int)sb.nblocks) {
@@ -685,11 +685,12 @@ struct HistcBody {
   }
 
   template <class SB>
-  static __device__ void run(const Args &a, SB &sb, unsigned char *lds, unsigned hint) {
+  static __device__ __forceinline__ void run(const Args &a, SB &sb, unsigned char *lds, unsigned hint) {
     // The original picks shared or global memory for the bins by what fits; so does the host here.
+    // (one global-memory instantiation, with the general bin formula: three copies of the loop
+    // keep the body small enough to be inlined at every call site of the fused kernel)
     if (hint & HINT_HIST_GLOBAL) {
-      if (hint & HINT_HIST_POW2) body<true, true>(a, sb, lds, hint);
-      else body<false, true>(a, sb, lds, hint);
+      body<false, true>(a, sb, lds, hint);
     } else if (hint & HINT_HIST_POW2) {
       body<true, false>(a, sb, lds, hint);
     } else {
