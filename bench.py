@@ -105,6 +105,10 @@ def time_tensor_pair(cfg, pair, steps, warmup, sweep, fused_only, rounds=5):
         # the two natives on two streams at once, the launch pattern of the reference's own traces
         res["t_two_streams_ms"] = statistics.median(
             [plan.time(4, pair.args1, pair.args2, 2, per) / per for _ in range(3)])
+        # the launch-bound preset: the same block shape, the build compiled for 8 waves per SIMD
+        lbplan = cfg.plan(cfg.find_fusion(pair.k1, pair.k2), "hfuse_lb")
+        res["t_fused_lb_ms"] = statistics.median(
+            [lbplan.time(3, pair.args1, pair.args2, 2, per) / per for _ in range(3)])
     res["split"] = label
     part = plan.partition
     res["fused_name"] = part.name.decode()
@@ -185,6 +189,8 @@ def run_search_pair(cfg, name, log2_a, log2_b, sweep, fused_only, iters=2):
     if not fused_only:
         res["t_vfuse_ms"] = cfg.plan(cfg.find_fusion(k1, k2), "vfuse").time(3, [a1], [a2], 0, 1, grid)
         res["t_two_streams_ms"] = base.time(4, [a1], [a2], 0, 1, grid)
+        lbplan = cfg.plan(cfg.find_fusion(k1, k2), "hfuse_lb")
+        res["t_fused_lb_ms"] = lbplan.time(3, [a1], [a2], 0, 1, grid_of(lbplan))
     res["split"] = label
     part = plan.partition
     res["fused_name"] = part.name.decode()

@@ -495,6 +495,7 @@ struct hf_plan {
   int barrier_mode;
   unsigned grid_override[2] = {0, 0};  // hf_plan_set_grids
   bool lending = true;                 // hf_plan_set_lending
+  int bounded = -1;                    // hf_plan_set_launch_bound: 0 / 1, -1 = by the preset
 };
 
 // ------------------------------------------------------------------ C-ABI
@@ -619,6 +620,7 @@ HF_API int hf_plan_create(const hf_config *cfg, int fusion_index, const char *pr
     return fail(HF_EINVAL, "search kernels are built for fused blocks of at most 512 threads");
   }
   if (f.lending >= 0) plan->lending = f.lending != 0;
+  if (f.launch_bound >= 0 && split_idx == HF_SPLIT_TABLE) plan->bounded = f.launch_bound;
   const bool b1 = body_has_barriers(plan->ids[0]), b2 = body_has_barriers(plan->ids[1]);
   // One barrier policy per pair: nothing to do when neither body synchronises;
   // an LDS-counter barrier scoped to the synchronising half otherwise.  (Both
@@ -694,6 +696,12 @@ HF_API int hf_plan_set_block(hf_plan *plan, int threads1, int threads2) {
 HF_API int hf_plan_set_lending(hf_plan *plan, int on) {
   if (!plan) return fail(HF_EINVAL, "null plan");
   plan->lending = on != 0;
+  return HF_OK;
+}
+
+HF_API int hf_plan_set_launch_bound(hf_plan *plan, int on) {
+  if (!plan) return fail(HF_EINVAL, "null plan");
+  plan->bounded = on < 0 ? -1 : (on != 0);
   return HF_OK;
 }
 
@@ -800,6 +808,12 @@ int do_launch_fused(const hf_plan *plan, const Prepared &p1, const Prepared &p2,
   if ((unsigned long long)std::max(exact, std::max(plan->grid_override[0], plan->grid_override[1])) * (g.d1 + g.d2) >
       0xFFFFFFFFull)
     return fail(HF_EINVAL, "grid_blocks * block threads must fit 32 bits (the bodies index work items with 32-bit counters)");
+  // The launch-bound presets run the register-bounded build whenever their block count asks for
+  // more waves per SIMD than the plain build's launch bound already guarantees.
+  const bool bounded = plan->bounded >= 0
+                           ? plan->bounded != 0
+                           : plan->preset->launch_bound &&
+                                 (unsigned long long)plan->part.launch_blocks * plan->part.launch_threads > 4ull * 256ull;
   hipError_t e;
   if (plan->preset->base_line) {
     // Vertical baseline: both kernels start at thread 0 of a block of max(d1, d2) threads.
@@ -808,8 +822,8 @@ int do_launch_fused(const hf_plan *plan, const Prepared &p1, const Prepared &p2,
     g.grid2 = p2.exact_grid ? exact : (grid_blocks > 0 ? (unsigned)grid_blocks : default_grid(p2, g.d2, block));
     const size_t lds = 4 * kBarrierWords + g.lds1 + g.lds2;
     const unsigned grid = std::max(g.grid1, g.grid2);
-    e = crypto ? launch_fused_crypto(plan->ids[0], plan->ids[1], MODE_VERTICAL, p1.blob, p2.blob, g, grid, lds, stream)
-               : launch_fused_dl(plan->ids[0], plan->ids[1], MODE_VERTICAL, p1.blob, p2.blob, g, grid, lds, stream);
+    e = crypto ? launch_fused_crypto(plan->ids[0], plan->ids[1], MODE_VERTICAL, bounded, p1.blob, p2.blob, g, grid, lds, stream)
+               : launch_fused_dl(plan->ids[0], plan->ids[1], MODE_VERTICAL, bounded, p1.blob, p2.blob, g, grid, lds, stream);
   } else if (plan->barrier_mode == HF_BARRIER_BLOCKIDX) {
     // Each kernel gets its own workgroups inside one launch.
     const unsigned block = std::max(g.d1, g.d2);
@@ -820,8 +834,8 @@ int do_launch_fused(const hf_plan *plan, const Prepared &p1, const Prepared &p2,
       g.grid2 = std::max(1u, (unsigned)grid_blocks - g.grid1);
     }
     const size_t lds = std::max(g.lds1, g.lds2);
-    e = crypto ? launch_fused_crypto(plan->ids[0], plan->ids[1], MODE_BLOCKIDX, p1.blob, p2.blob, g, g.grid1 + g.grid2, lds, stream)
-               : launch_fused_dl(plan->ids[0], plan->ids[1], MODE_BLOCKIDX, p1.blob, p2.blob, g, g.grid1 + g.grid2, lds, stream);
+    e = crypto ? launch_fused_crypto(plan->ids[0], plan->ids[1], MODE_BLOCKIDX, false, p1.blob, p2.blob, g, g.grid1 + g.grid2, lds, stream)
+               : launch_fused_dl(plan->ids[0], plan->ids[1], MODE_BLOCKIDX, false, p1.blob, p2.blob, g, g.grid1 + g.grid2, lds, stream);
   } else {
     // One grid for both halves.  When the caller names it, both halves stride over all of it
     // (a kernel whose grid fixes its work, ethash, always does); otherwise each half strides
@@ -848,8 +862,8 @@ int do_launch_fused(const hf_plan *plan, const Prepared &p1, const Prepared &p2,
     const unsigned grid = std::max(g.grid1, g.grid2);
     const size_t lds = 4 * kBarrierWords + g.lds1 + g.lds2;
     const FuseMode mode = plan->barrier_mode == HF_BARRIER_MATCHED ? MODE_MATCHED : MODE_HFUSE;
-    e = crypto ? launch_fused_crypto(plan->ids[0], plan->ids[1], mode, p1.blob, p2.blob, g, grid, lds, stream)
-               : launch_fused_dl(plan->ids[0], plan->ids[1], mode, p1.blob, p2.blob, g, grid, lds, stream);
+    e = crypto ? launch_fused_crypto(plan->ids[0], plan->ids[1], mode, bounded, p1.blob, p2.blob, g, grid, lds, stream)
+               : launch_fused_dl(plan->ids[0], plan->ids[1], mode, bounded, p1.blob, p2.blob, g, grid, lds, stream);
   }
   if (e == hipErrorNotSupported) return fail(HF_EUNSUPPORTED, "this pair / barrier mode is not built");
   if (e != hipSuccess) return hip_fail(e, "fused launch");

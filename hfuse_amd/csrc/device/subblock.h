@@ -94,8 +94,9 @@ __global__ __launch_bounds__(T) void native_kernel(typename K::Args a, unsigned 
 // divergence.  MATCHED: both bodies execute the same number of barriers, so
 // they may share the hardware barrier; otherwise a body that synchronises
 // uses its own LDS counter.
-template <class K1, class K2, int T, bool MATCHED>
-__global__ __launch_bounds__(T) void fused_kernel(typename K1::Args a1, typename K2::Args a2, FuseGeom g) {
+template <class K1, class K2, bool MATCHED>
+__device__ __forceinline__ void fused_block(const typename K1::Args &a1, const typename K2::Args &a2,
+                                            const FuseGeom &g) {
   extern __shared__ __align__(16) unsigned char smem[];
   unsigned *bars = reinterpret_cast<unsigned *>(smem);
   const unsigned tid = threadIdx.x;
@@ -147,6 +148,25 @@ __global__ __launch_bounds__(T) void fused_kernel(typename K1::Args a1, typename
   }
 }
 
+template <class K1, class K2, int T, bool MATCHED>
+__global__ __launch_bounds__(T) void fused_kernel(typename K1::Args a1, typename K2::Args a2, FuseGeom g) {
+  fused_block<K1, K2, MATCHED>(a1, a2, g);
+}
+
+// The launch-bound presets (hfuse_lb, vfuse_lb).  The reference prints
+// `__launch_bounds__(T, B)` with B = min_k(regfile / Reg_k / size_k) capped by the resident
+// thread limit (lib/KernelFuser/KernelPrinter.cpp:44-66), i.e. it makes the compiler keep the
+// fused kernel's registers low enough for the occupancy the natives had.  The gfx950 form of
+// that request is a waves-per-SIMD bound: this build of each fused kernel is compiled for
+// kBoundedWaves waves per SIMD (at most 512 / 8 = 64 vector registers), spilling if it must.
+constexpr int kBoundedWaves = 8;
+
+template <class K1, class K2, int T, bool MATCHED>
+__global__ __launch_bounds__(T) __attribute__((amdgpu_waves_per_eu(kBoundedWaves, kBoundedWaves)))
+void fused_kernel_lb(typename K1::Args a1, typename K2::Args a2, FuseGeom g) {
+  fused_block<K1, K2, MATCHED>(a1, a2, g);
+}
+
 // Fallback when the halves cannot share a workgroup: workgroups [0, grid1) run
 // kernel 1 and [grid1, grid1+grid2) run kernel 2, each with the whole
 // workgroup's hardware barrier.  The block is max(d1, d2) threads; waves beyond
@@ -172,8 +192,9 @@ __global__ __launch_bounds__(T) void blockidx_kernel(typename K1::Args a1, typen
 // and the same threads run kernel 1's body and then kernel 2's.  A body that synchronises
 // uses its LDS arrival counter, because the threads beyond its own size are still alive
 // (they wait for, or already run, the other body) and must not be waited for.
-template <class K1, class K2, int T>
-__global__ __launch_bounds__(T) void vertical_kernel(typename K1::Args a1, typename K2::Args a2, FuseGeom g) {
+template <class K1, class K2>
+__device__ __forceinline__ void vertical_block(const typename K1::Args &a1, const typename K2::Args &a2,
+                                               const FuseGeom &g) {
   extern __shared__ __align__(16) unsigned char smem[];
   unsigned *bars = reinterpret_cast<unsigned *>(smem);
   const unsigned tid = threadIdx.x, bid = blockIdx.x;
@@ -192,6 +213,17 @@ __global__ __launch_bounds__(T) void vertical_kernel(typename K1::Args a1, typen
     SubBlock<B2> sb{tid, g.d2, bid, g.grid2, bars + 1, 0, bid * g.d2, g.grid2 * g.d2};
     K2::run(a2, sb, smem + 4 * kBarrierWords + g.lds1, g.hint2);
   }
+}
+
+template <class K1, class K2, int T>
+__global__ __launch_bounds__(T) void vertical_kernel(typename K1::Args a1, typename K2::Args a2, FuseGeom g) {
+  vertical_block<K1, K2>(a1, a2, g);
+}
+
+template <class K1, class K2, int T>
+__global__ __launch_bounds__(T) __attribute__((amdgpu_waves_per_eu(kBoundedWaves, kBoundedWaves)))
+void vertical_kernel_lb(typename K1::Args a1, typename K2::Args a2, FuseGeom g) {
+  vertical_block<K1, K2>(a1, a2, g);
 }
 
 }  // namespace hfuse

@@ -166,6 +166,11 @@ bool parse_config(const char *fusion_yaml, const char *kernels_yaml, Config &cfg
         else if (ln->kind == YamlNode::Scalar && (ln->scalar == "false" || ln->scalar == "0")) f.lending = 0;
         else { err = "fusion list: " + at(*ln) + "'Lending' must be true or false"; return false; }
       }
+      if (const YamlNode *lb = n.get("LaunchBound")) {
+        if (lb->kind == YamlNode::Scalar && (lb->scalar == "true" || lb->scalar == "1")) f.launch_bound = 1;
+        else if (lb->kind == YamlNode::Scalar && (lb->scalar == "false" || lb->scalar == "0")) f.launch_bound = 0;
+        else { err = "fusion list: " + at(*lb) + "'LaunchBound' must be true or false"; return false; }
+      }
       if (const YamlNode *bn = n.get("Barrier")) {
         static const char *const kModes[] = {"none", "matched", "subset", "blockidx"};  // HF_BARRIER_* order
         for (int m = 0; m < 4; m++)
@@ -177,7 +182,7 @@ bool parse_config(const char *fusion_yaml, const char *kernels_yaml, Config &cfg
       }
       for (auto &kv : n.map)
         if (kv.first != "File" && kv.first != "Kernels" && kv.first != "Split" && kv.first != "Threads" &&
-            kv.first != "Lending" && kv.first != "Barrier") {
+            kv.first != "Lending" && kv.first != "Barrier" && kv.first != "LaunchBound") {
           err = "fusion list: " + at(kv.second) + "unknown key '" + kv.first + "'";
           return false;
         }

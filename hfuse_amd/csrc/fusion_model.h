@@ -31,6 +31,7 @@ struct FusionRow {
   uint32_t split = 0;    // optional `Split:` key: threads of kernel 1 when the caller asks for the table split
   uint32_t threads = 0;  // optional `Threads:` key: threads of the whole fused block (needs Split)
   int lending = -1;      // optional `Lending:` key: 0 / 1 switch wave lending off / on, -1 = library default
+  int launch_bound = -1; // optional `LaunchBound:` key: 0 / 1 pick the plain / register-bounded build, -1 = the preset's
   int barrier = -1;      // optional `Barrier:` key: an HF_BARRIER_* mode, -1 = library default
 };
 

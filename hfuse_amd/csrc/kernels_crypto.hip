@@ -19,20 +19,29 @@ hipError_t native(const void *args, unsigned hint, unsigned grid, unsigned block
 }
 
 template <class K1, class K2>
-hipError_t pair(FuseMode mode, const void *a1, const void *a2, const FuseGeom &g, unsigned grid, size_t lds,
+hipError_t pair(FuseMode mode, bool bounded, const void *a1, const void *a2, const FuseGeom &g, unsigned grid, size_t lds,
                 hipStream_t s) {
   const auto &x1 = *static_cast<const typename K1::Args *>(a1);
   const auto &x2 = *static_cast<const typename K2::Args *>(a2);
   if (g.d1 + g.d2 > (unsigned)kCryptoBlock) return hipErrorNotSupported;
   switch (mode) {
     case MODE_HFUSE:
-      hipLaunchKernelGGL((fused_kernel<K1, K2, kCryptoBlock, false>), dim3(grid), dim3(g.d1 + g.d2), lds, s, x1, x2,
-                         g);
+      if (bounded)
+        hipLaunchKernelGGL((fused_kernel_lb<K1, K2, kCryptoBlock, false>), dim3(grid), dim3(g.d1 + g.d2), lds, s, x1,
+                           x2, g);
+      else
+        hipLaunchKernelGGL((fused_kernel<K1, K2, kCryptoBlock, false>), dim3(grid), dim3(g.d1 + g.d2), lds, s, x1, x2,
+                           g);
       break;
     case MODE_MATCHED:
       return hipErrorNotSupported;  // none of the searches has a barrier
     case MODE_VERTICAL:
-      hipLaunchKernelGGL((vertical_kernel<K1, K2, kCryptoBlock>), dim3(grid), dim3(g.d1 > g.d2 ? g.d1 : g.d2), lds, s, x1, x2, g);
+      if (bounded)
+        hipLaunchKernelGGL((vertical_kernel_lb<K1, K2, kCryptoBlock>), dim3(grid), dim3(g.d1 > g.d2 ? g.d1 : g.d2), lds,
+                           s, x1, x2, g);
+      else
+        hipLaunchKernelGGL((vertical_kernel<K1, K2, kCryptoBlock>), dim3(grid), dim3(g.d1 > g.d2 ? g.d1 : g.d2), lds, s,
+                           x1, x2, g);
       break;
     case MODE_BLOCKIDX:
       hipLaunchKernelGGL((blockidx_kernel<K1, K2, kCryptoBlock>), dim3(grid), dim3(g.d1 > g.d2 ? g.d1 : g.d2), lds,
@@ -56,10 +65,10 @@ hipError_t launch_native_crypto(KernelId k, const void *args, unsigned hint, uns
 }
 
 #define HF_PAIR(A, KA, B, KB)                                                     \
-  if (k1 == A && k2 == B) return pair<KA, KB>(mode, a1, a2, g, grid, lds, s);     \
-  if (k1 == B && k2 == A) return pair<KB, KA>(mode, a1, a2, g, grid, lds, s);
+  if (k1 == A && k2 == B) return pair<KA, KB>(mode, bounded, a1, a2, g, grid, lds, s);     \
+  if (k1 == B && k2 == A) return pair<KB, KA>(mode, bounded, a1, a2, g, grid, lds, s);
 
-hipError_t launch_fused_crypto(KernelId k1, KernelId k2, FuseMode mode, const void *a1, const void *a2,
+hipError_t launch_fused_crypto(KernelId k1, KernelId k2, FuseMode mode, bool bounded, const void *a1, const void *a2,
                                const FuseGeom &g, unsigned grid, size_t lds, hipStream_t s) {
   HF_PAIR(K_ETHASH, EthashBody, K_BLAKE2B, CcminerBlake2bBody)
   HF_PAIR(K_SHA256D, Sha256dBody, K_ETHASH, EthashBody)

@@ -33,10 +33,11 @@ hipError_t launch_native_dl(KernelId k, const void *dev_args, unsigned hint, uns
 hipError_t launch_native_crypto(KernelId k, const void *dev_args, unsigned hint, unsigned grid, unsigned block,
                                 size_t lds, hipStream_t stream);
 
-// Returns hipErrorNotSupported when the pair is not instantiated.
-hipError_t launch_fused_dl(KernelId k1, KernelId k2, FuseMode mode, const void *a1, const void *a2,
+// Returns hipErrorNotSupported when the pair is not instantiated.  `bounded` selects the
+// register-bounded build of the fused / vertical kernel (the launch-bound presets).
+hipError_t launch_fused_dl(KernelId k1, KernelId k2, FuseMode mode, bool bounded, const void *a1, const void *a2,
                            const FuseGeom &g, unsigned grid, size_t lds, hipStream_t stream);
-hipError_t launch_fused_crypto(KernelId k1, KernelId k2, FuseMode mode, const void *a1, const void *a2,
+hipError_t launch_fused_crypto(KernelId k1, KernelId k2, FuseMode mode, bool bounded, const void *a1, const void *a2,
                                const FuseGeom &g, unsigned grid, size_t lds, hipStream_t stream);
 
 hipError_t launch_fill_splitmix64(unsigned long long *dst, unsigned long long nwords, unsigned long long seed,

@@ -115,6 +115,10 @@ class Plan:
     def set_lending(self, on: bool) -> None:
         check(L.lib().hf_plan_set_lending(self._h, int(on)))
 
+    def set_launch_bound(self, on) -> None:
+        """True / False: run the register-bounded / the plain build; None: by the preset."""
+        check(L.lib().hf_plan_set_launch_bound(self._h, -1 if on is None else int(bool(on))))
+
     def local_index(self, half: int, tid: int):
         out = L.Dim3()
         check(L.lib().hf_plan_local_index(self._h, half, tid, C.byref(out)))

@@ -5,13 +5,14 @@ The reference generates one fused kernel per split of the enumeration 128*(n+1) 
 Here every split is a launch-time choice of the same compiled kernel, so the sweep is a loop of
 timed launches: block shapes (threads of kernel 1, threads of kernel 2) in wavefront multiples,
 wave lending on and off, and the barrier modes legal for the pair.  The winner is written back
-into the fusion list as the `Split:` / `Threads:` / `Lending:` / `Barrier:` keys the library applies when a
-plan is created with the table split.
+into the fusion list as the `Split:` / `Threads:` / `Lending:` / `Barrier:` / `LaunchBound:` keys
+the library applies when a plan is created with the table split.
 
 The register-cap half of the reference's experiments (its *_lb presets, `Reg` bound per
-kernel) has no launch-time counterpart: a gfx950 kernel's VGPR budget follows from its launch
-bound at compile time.  What a launch can still choose is how many blocks share a CU, which is
-the `grids` dimension of the sweep (blocks per CU for each half of the fused grid).
+kernel): a gfx950 kernel's VGPR budget is fixed at compile time, so the library carries two
+builds of every fused kernel, plain and bounded to 8 waves per SIMD, and the sweep times the
+finalists in both.  How many blocks share a CU is the `grids` dimension of the sweep (blocks
+per CU for each half of the fused grid).
 
     python -m hfuse_amd.tuner --out tuned_fusion.yaml            # all shipped tensor pairs
     python -m hfuse_amd.tuner --only Im2ColMaxPool,SummaryMaxpool --out tuned.yaml
@@ -41,6 +42,7 @@ class Candidate:
     lending: bool = True
     barrier_mode: Optional[int] = None   # None: the library's choice for the pair
     grids: Tuple[int, int] = (0, 0)      # (0, 0): the library's grids
+    bounded: bool = False                # the register-bounded build (the reference's *_lb presets)
 
     def label(self) -> str:
         s = f"{self.threads1}+{self.threads2}"
@@ -50,6 +52,8 @@ class Candidate:
             s += f" {BARRIER_NAMES[self.barrier_mode]}"
         if self.grids != (0, 0):
             s += f" grids{self.grids[0]}x{self.grids[1]}"
+        if self.bounded:
+            s += " lb"
         return s
 
 
@@ -103,6 +107,7 @@ def _make_plan(cfg: H.Config, fusion_index: int, c: Candidate) -> H.Plan:
         plan.set_barrier_mode(c.barrier_mode)
     if c.grids != (0, 0):
         plan.set_grids(*c.grids)
+    plan.set_launch_bound(c.bounded)
     return plan
 
 
@@ -110,13 +115,14 @@ def tune(cfg: H.Config, fusion_index: int, args1: Sequence, args2: Sequence, *,
          blocks: Optional[Sequence[Tuple[int, int]]] = None, lending: Sequence[bool] = (True, False),
          barrier_modes: Sequence[Optional[int]] = (None,), grids: Sequence[Tuple[int, int]] = ((0, 0),),
          probe_iters: int = 20, final_iters: int = 100, finalists: int = 4, warmup: int = 3,
-         grid_blocks=0, verbose: bool = False) -> TuneResult:
+         grid_blocks=0, launch_bound: bool = True, verbose: bool = False) -> TuneResult:
     """Sweep the candidates of one pair on the caller's argument sets and return the fastest.
 
     args1[i] / args2[i] are argument structs of independent buffer sets the timed launches rotate
     through (hf_time_pair).  Every candidate gets `probe_iters` launches; the `finalists` fastest
     are timed again over `final_iters` launches in three interleaved rounds, together with the
-    back-to-back native launches and the untuned table split, and the median decides.
+    back-to-back native launches and the untuned table split, and the median decides.  With
+    `launch_bound` each finalist also runs in the register-bounded build.
 
     `grid_blocks` is the launch grid (0: the library's) or a function (threads1, threads2) -> grid
     for kernels whose grid fixes their work: Ethash scans grid * its-threads nonces, so a fair
@@ -141,6 +147,11 @@ def tune(cfg: H.Config, fusion_index: int, args1: Sequence, args2: Sequence, *,
         raise RuntimeError(f"no legal candidate for {k1} + {k2}")
     probed.sort(key=lambda r: r[0])
     final = probed[:max(1, finalists)]
+    if launch_bound:
+        import dataclasses
+        for t, c, _ in list(final):
+            twin = dataclasses.replace(c, bounded=True)
+            final.append((t, twin, _make_plan(cfg, fusion_index, twin)))
     # Untuned reference point: the kernel table's own split, whatever the fusion entry says.
     base_cfg_plan = cfg.plan(fusion_index, "hfuse", 0)
     d1 = cfg.kernel(k1).block_dim
@@ -163,15 +174,17 @@ def tune(cfg: H.Config, fusion_index: int, args1: Sequence, args2: Sequence, *,
     # Timings this close are the same speed: among them prefer the library's defaults
     # (lending on, the pair's own barrier design) so that noise does not write keys.
     near = [(t, i) for t, i in med if t <= med[0][0] * 1.005]
-    t_best, ibest = min(near, key=lambda r: ((not final[r[1]][1].lending) + (final[r[1]][1].barrier_mode is not None), r[0]))
+    t_best, ibest = min(near, key=lambda r: ((not final[r[1]][1].lending) + (final[r[1]][1].barrier_mode is not None)
+                                             + final[r[1]][1].bounded, r[0]))
     return TuneResult(file=file, kernels=(k1, k2), best=final[ibest][1], t_best_ms=t_best,
                       t_table_ms=statistics.median(s_table) if s_table else float("nan"),
                       t_b2b_ms=statistics.median(s_b2b),
-                      table=[(c.label(), t) for t, c, _ in probed])
+                      table=[(c.label(), t) for t, c, _ in probed] +
+                            [(final[i][1].label(), t) for t, i in med if final[i][1].bounded])
 
 
 # ------------------------------------------------------------------ fusion list rewriting
-_TUNED_KEY = re.compile(r"^\s+(Split|Threads|Lending|Barrier)\s*:")
+_TUNED_KEY = re.compile(r"^\s+(Split|Threads|Lending|Barrier|LaunchBound)\s*:")
 BARRIER_NAMES = {L.HF_BARRIER_NONE: "none", L.HF_BARRIER_MATCHED: "matched", L.HF_BARRIER_SUBSET: "subset",
                  L.HF_BARRIER_BLOCKIDX: "blockidx"}
 
@@ -202,6 +215,8 @@ def apply_to_fusion_yaml(text: str, tuned: dict) -> str:
                     entry.append("  Lending: false")
                 if c.barrier_mode is not None:
                     entry.append(f"  Barrier: {BARRIER_NAMES[c.barrier_mode]}")
+                if c.bounded:
+                    entry.append("  LaunchBound: true")
             entry.extend(tail)
         out.extend(entry)
     if not starts:

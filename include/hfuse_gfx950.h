@@ -75,13 +75,14 @@ typedef struct {
  * and a string-keyed map of kernel rows.  `kernels_yaml` may also be the older
  * per-pair form, a bare sequence of rows (configs/im2col_maxpool.yaml); then
  * `fusion_yaml` may be NULL and the single fusion is that list in order.
- * Four keys beyond the reference's schema are accepted in a fusion entry
+ * Five keys beyond the reference's schema are accepted in a fusion entry
  * (the split tuner writes them): `Split: <threads>`, a tuned default for
  * kernel 1's share of the block, and `Threads: <threads>`, a tuned size of the
  * whole fused block (kernel 2 gets Threads - Split); both apply when a plan is
  * created with HF_SPLIT_TABLE.  `Lending: true|false` sets the plan's default
  * for hf_plan_set_lending and `Barrier: none|matched|subset|blockidx` the one
- * for hf_plan_set_barrier_mode (an illegal mode fails hf_plan_create).
+ * for hf_plan_set_barrier_mode (an illegal mode fails hf_plan_create);
+ * `LaunchBound: true|false` the one for hf_plan_set_launch_bound.
  */
 HF_API int hf_config_load_text(const char *fusion_yaml, const char *kernels_yaml, hf_config **out);
 HF_API int hf_config_load_files(const char *fusion_path, const char *kernels_path, hf_config **out);
@@ -127,8 +128,8 @@ enum {
  *               The hfuse presets partition the block's threads between the two
  *               kernels; the vfuse presets are the reference's baseline in which
  *               the same threads run kernel 1 and then kernel 2 (block =
- *               max(d1, d2)).  The _lb variants differ only in the reported
- *               launch_blocks hint.
+ *               max(d1, d2)).  The _lb variants report the launch_blocks hint
+ *               and run the register-bounded build (hf_plan_set_launch_bound).
  *   split_idx : the reference's enumeration index n (Split = 128*(n+1) threads
  *               for kernel 1, main.cpp:216-227); HF_SPLIT_TABLE keeps the
  *               YAML's BlockDim as the split; HF_SPLIT_EXECTIME re-splits in
@@ -171,6 +172,20 @@ HF_API int hf_plan_set_block(hf_plan *plan, int threads1, int threads2);
  * once, which is what the reference's generated kernel does.  Results are identical.
  */
 HF_API int hf_plan_set_lending(hf_plan *plan, int on);
+/*
+ * Which build of the fused (or vertical) kernel a launch runs.  The reference's *_lb presets
+ * print `__launch_bounds__(T, B)` with B = min_k(regfile / Reg_k / size_k), capped by the
+ * resident-thread limit (lib/KernelFuser/KernelPrinter.cpp:44-66), so that the compiler keeps
+ * the fused kernel's registers within the occupancy the natives had.  On gfx950 that request
+ * is a waves-per-SIMD bound, fixed at compile time: every pair is built twice, plain (bounded
+ * only by its launch bound of 1024 or 512 threads) and register-bounded for 8 waves per SIMD
+ * (at most 64 vector registers, spilling to a private stack if it must).
+ *   on = 1 / 0 : run the bounded / the plain build whatever the preset;
+ *   on < 0     : by the preset (default): hfuse_lb and vfuse_lb run the bounded build when
+ *                launch_blocks * launch_threads asks for more than 4 waves per SIMD.
+ * The blockIdx fallback has no bounded build.  Results are identical; only the time differs.
+ */
+HF_API int hf_plan_set_launch_bound(hf_plan *plan, int on);
 HF_API int hf_plan_partition(const hf_plan *plan, hf_partition *out);
 /* Number of variants the reference's split loop would print (main.cpp:221-223). */
 HF_API int hf_plan_num_splits(const hf_config *cfg, int fusion_index);

@@ -224,6 +224,20 @@ def test_every_shipped_search_pair(cuda, cfg):
             sync()
             assert H.read_search_results(r1) == native[k1], (k1, k2)
             assert H.read_search_results(r2) == native[k2], (k1, k2)
+            # the register-bounded builds (8 waves per SIMD; these spill): same found sets
+            for preset in ("hfuse", "vfuse"):
+                r1, a1 = _search_pair_args(cuda, k1, count, 42)
+                r2, a2 = _search_pair_args(cuda, k2, count, 42)
+                if k1.endswith("blake2b_gpu_hash"):
+                    a1 = H.blake2b_args(r1, count, 42, EASY10)
+                if k2.endswith("blake2b_gpu_hash"):
+                    a2 = H.blake2b_args(r2, count, 42, EASY10)
+                plan = cfg.plan(i, preset)
+                plan.set_launch_bound(True)
+                plan.launch(a1, a2, grid_blocks=grid)
+                sync()
+                assert H.read_search_results(r1) == native[k1], (k1, k2, preset, "bounded")
+                assert H.read_search_results(r2) == native[k2], (k1, k2, preset, "bounded")
             n += 1
     assert n == 7
 

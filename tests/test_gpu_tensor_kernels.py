@@ -550,6 +550,15 @@ def test_every_shipped_tensor_pair(cuda, cfg):
             sync()
             a.check()
             b.check()
+            # the register-bounded build of the same pair, horizontal and vertical
+            for preset in ("hfuse", "vfuse"):
+                plan = cfg.plan(i, preset)
+                plan.set_launch_bound(True)
+                a, b = makers[k1](), makers[k2]()
+                plan.launch(a.args, b.args)
+                sync()
+                a.check()
+                b.check()
             n += 1
     assert n == 11  # the ten pairs of the reference list plus bn+upsample in benchmark order
 

@@ -12,6 +12,11 @@ import pytest
 from hfuse_amd import _lib
 from hfuse_amd.codeobj import kernel_resources, offload_bundles, short_name
 
+# The launch-bound presets' builds are compiled for 8 waves per SIMD and may spill: that is their point.
+def bounded(r):
+    return "_lb<" in short_name(r.name)
+
+
 TENSOR = ("Im2col", "MaxPool", "BnStats", "UpsampleNearest", "UpsampleBilinear", "Histc")
 SEARCH = ("Sha256d", "Blake2b", "Ethash")
 
@@ -33,26 +38,26 @@ def test_every_kernel_family_is_present(rows):
     names = [short_name(r.name) for r in rows]
     for body in TENSOR + SEARCH:
         assert any(n.startswith("native_kernel<" + body) for n in names), body
-    for kind in ("fused_kernel<", "vertical_kernel<", "blockidx_kernel<"):
+    for kind in ("fused_kernel<", "vertical_kernel<", "blockidx_kernel<", "fused_kernel_lb<", "vertical_kernel_lb<"):
         assert sum(n.startswith(kind) for n in names) >= 20, kind
 
 
 def test_no_vector_spills_and_no_dynamic_stack(rows):
     # (scalar registers may spill: they go to lanes of a vector register, not to memory)
-    bad = [short_name(r.name) for r in rows if r.vgpr_spills or r.dynamic_stack]
+    bad = [short_name(r.name) for r in rows if (r.vgpr_spills and not bounded(r)) or r.dynamic_stack]
     assert not bad, bad
 
 
 def test_tensor_kernels_have_no_private_stack(rows):
     bad = [(short_name(r.name), r.private_bytes) for r in rows
-           if r.private_bytes and not any(s in r.name for s in SEARCH)]
+           if r.private_bytes and not bounded(r) and not any(s in r.name for s in SEARCH)]
     assert not bad, bad
 
 
 def test_search_kernels_only_carry_the_record_helper_stack(rows):
     # the rarely taken "record a hit" helper is deliberately a call; its frame is 48 bytes
     bad = [(short_name(r.name), r.private_bytes) for r in rows
-           if any(s in r.name for s in SEARCH) and r.private_bytes > 64]
+           if any(s in r.name for s in SEARCH) and not bounded(r) and r.private_bytes > 64]
     assert not bad, bad
 
 
@@ -75,6 +80,13 @@ def test_fusing_never_halves_occupancy(rows):
         assert r.vgpr <= 1.25 * need + 8, (short_name(r.name), r.vgpr, need)
         checked += 1
     assert checked >= 20
+
+
+def test_bounded_builds_fit_eight_waves_per_simd(rows):
+    lb = [r for r in rows if bounded(r)]
+    assert len(lb) >= 40
+    bad = [(short_name(r.name), r.vgpr + r.agpr) for r in lb if r.vgpr + r.agpr > 64]
+    assert not bad, bad
 
 
 def test_cli_prints_a_table(capsys):

@@ -64,7 +64,7 @@ def test_stripping_every_entry_gives_the_untuned_list():
     n = fusion.count("- File:")
     clean = T.apply_to_fusion_yaml(fusion, {i: None for i in range(n)})
     body = [ln for ln in clean.splitlines() if not ln.lstrip().startswith("#")]
-    assert not any(ln.split(":")[0].strip() in ("Split", "Threads", "Lending", "Barrier") for ln in body)
+    assert not any(ln.split(":")[0].strip() in ("Split", "Threads", "Lending", "Barrier", "LaunchBound") for ln in body)
     cfg = H.Config(clean, kernels)
     assert cfg.fusions() == H.Config(fusion, kernels).fusions()
     p = cfg.plan(cfg.find_fusion("kernelHistogram1D", "MaxPoolForward")).partition
@@ -96,6 +96,23 @@ def test_lending_key():
     assert e.value.code == L.HF_EPARSE and "Lending" in e.value.message
 
 
+def test_launch_bound_key():
+    _, kernels = shipped()
+    base = "- File: a\n  Kernels:\n    - im2col_kernel\n    - MaxPoolForward\n"
+    H.Config(base + "  LaunchBound: true\n", kernels).plan(0)
+    H.Config(base + "  LaunchBound: false\n", kernels).plan(0, "hfuse_lb")
+    with pytest.raises(hfuse_amd.HfuseError) as e:
+        H.Config(base + "  LaunchBound: 8\n", kernels)
+    assert e.value.code == L.HF_EPARSE and "LaunchBound" in e.value.message
+    text = T.apply_to_fusion_yaml(base, {0: T.Candidate(256, 256, bounded=True)})
+    assert text == base + "  Split: 256\n  Threads: 512\n  LaunchBound: true\n"
+    assert T.apply_to_fusion_yaml(text, {0: T.Candidate(256, 256)}) == base + "  Split: 256\n  Threads: 512\n"
+    assert T.Candidate(128, 64, bounded=True).label() == "128+64 lb"
+    plan = H.Config(base, kernels).plan(0)
+    for on in (True, False, None):
+        plan.set_launch_bound(on)
+
+
 @pytest.mark.gpu
 def test_small_sweep_and_tuned_launch(cuda):
     from test_gpu_tensor_kernels import Im2col, MaxPool, sync
@@ -107,7 +124,8 @@ def test_small_sweep_and_tuned_launch(cuda):
     shapes = [(128, 128), (256, 256), (512, 256), (256, 512)]
     r = T.tune(cfg, i, [t.args for t in a], [t.args for t in b], blocks=shapes, probe_iters=5, final_iters=10, finalists=2)
     assert (r.best.threads1, r.best.threads2) in shapes
-    assert len(r.table) == 8 and r.t_best_ms > 0 and r.t_b2b_ms > 0 and r.t_table_ms > 0
+    # 4 shapes x lending on / off, plus the two finalists again in the register-bounded build
+    assert len(r.table) == 10 and sum(lab.endswith(" lb") for lab, _ in r.table) == 2 and r.t_best_ms > 0 and r.t_b2b_ms > 0 and r.t_table_ms > 0
     for t in a + b:   # the sweep's own launches wrote correct results
         sync()
         t.check()
