@@ -14,6 +14,8 @@ block shape instead:
     fused_kernel<XBody, YBody, .., 0>    HF   horizontally fused, tagged with the workgroup size
     fused_kernel<XBody, YBody, .., 1>    HF+M the same with the shared hardware barrier
     blockidx_kernel<XBody, YBody, ...>   BI   block-index partition
+    fused_kernel_lb / vertical_kernel_lb HF-LB, HF+M-LB, VF-LB: the register-bounded builds
+                                         (the reference's hfuse_lb / vfuse_lb presets)
 
 Input: the `*_kernel_trace.csv` of `rocprofv3 --kernel-trace --output-format csv` and, for the
 metric table, any number of `*_counter_collection.csv` files of `rocprofv3 --pmc ...` runs of the
@@ -54,20 +56,20 @@ SHORT = {
     "kernelHistogram1D": "Hist", "ethash_search": "Ethash", "sha256d_gpu_hash_shared": "SHA256",
     "sia_blake2b_gpu_hash": "Blake2B", "blake2b_gpu_hash": "Blake2B(cc)",
 }
-TAG_ORDER = ("ST", "VF", "HF", "HF+M", "BI")
+TAG_ORDER = ("ST", "VF", "VF-LB", "HF", "HF-LB", "HF+M", "HF+M-LB", "BI")
 
-_TEMPLATE = re.compile(r"hfuse::(native_kernel|fused_kernel|vertical_kernel|blockidx_kernel)<(.*)>\(")
+_TEMPLATE = re.compile(r"hfuse::(native_kernel|fused_kernel_lb|fused_kernel|vertical_kernel_lb|vertical_kernel|blockidx_kernel)<(.*)>\(")
 _BODY = re.compile(r"hfuse::(\w+Body(?:<[^<>]*>)?)")
 
 
 @dataclass(frozen=True)
 class KernelKey:
-    tag: str                       # ST, VF, HF, HF+M, BI
+    tag: str                       # one of TAG_ORDER
     kernels: Tuple[str, ...]       # one YAML kernel name (ST) or two
     block: int                     # workgroup size of the launch
 
     def label(self) -> str:
-        return self.tag if self.tag in ("ST", "VF") else f"{self.tag}@{self.block}"
+        return self.tag if self.tag in ("ST", "VF", "VF-LB") else f"{self.tag}@{self.block}"
 
 
 def parse_kernel_name(name: str) -> Optional[Tuple[str, Tuple[str, ...]]]:
@@ -83,12 +85,13 @@ def parse_kernel_name(name: str) -> Optional[Tuple[str, Tuple[str, ...]]]:
         return "ST", (bodies[0],)
     if len(bodies) != 2:
         return None
-    if kind == "vertical_kernel":
-        return "VF", tuple(bodies)
+    lb = "-LB" if kind.endswith("_lb") else ""
+    if kind.startswith("vertical_kernel"):
+        return "VF" + lb, tuple(bodies)
     if kind == "blockidx_kernel":
         return "BI", tuple(bodies)
     matched = params.rstrip().endswith("true")
-    return ("HF+M" if matched else "HF"), tuple(bodies)
+    return ("HF+M" if matched else "HF") + lb, tuple(bodies)
 
 
 @dataclass

@@ -19,6 +19,11 @@ def test_parse_kernel_name():
     assert A.parse_kernel_name(F.format(a="BnStatsBody", b="HistcBody", m="true"))[0] == "HF+M"
     assert A.parse_kernel_name(V.format(a="EthashBody", b="Blake2bBody<4, false>")) == ("VF", ("ethash_search", "sia_blake2b_gpu_hash"))
     assert A.parse_kernel_name(B.format(a="Blake2bBody<9, true>", b="Sha256dBody")) == ("BI", ("blake2b_gpu_hash", "sha256d_gpu_hash_shared"))
+    # the register-bounded builds (the reference's *_lb presets)
+    assert A.parse_kernel_name(F.replace("fused_kernel<", "fused_kernel_lb<").format(a="HistcBody", b="MaxPoolBody", m="false"))[0] == "HF-LB"
+    assert A.parse_kernel_name(F.replace("fused_kernel<", "fused_kernel_lb<").format(a="HistcBody", b="BnStatsBody", m="true"))[0] == "HF+M-LB"
+    assert A.parse_kernel_name(V.replace("vertical_kernel<", "vertical_kernel_lb<").format(a="Im2colBody", b="MaxPoolBody")) == ("VF-LB", ("im2col_kernel", "MaxPoolForward"))
+    assert A.KernelKey("HF-LB", ("a", "b"), 512).label() == "HF-LB@512" and A.KernelKey("VF-LB", ("a", "b"), 512).label() == "VF-LB"
     assert A.parse_kernel_name("void at::native::vectorized_elementwise_kernel<4, Foo>(int)") is None
     assert A.parse_kernel_name("void hfuse::(anonymous namespace)::copy_f32_kernel(float const*, float*, unsigned long long)") is None
     # every body the library instantiates has a YAML name
