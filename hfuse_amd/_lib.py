@@ -11,14 +11,14 @@ import os
 _HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(_HERE, "libhfuse_gfx950.so")
 
-HF_OK, HF_EINVAL, HF_EPARSE, HF_ENOTFOUND, HF_EUNSUPPORTED, HF_EHIP, HF_EIO = 0, -1, -2, -3, -4, -5, -6
+HF_OK, HF_EINVAL, HF_EPARSE, HF_ENOTFOUND, HF_EUNSUPPORTED, HF_EHIP, HF_EIO, HF_ENOMEM = 0, -1, -2, -3, -4, -5, -6, -7
 HF_BARRIER_NONE, HF_BARRIER_MATCHED, HF_BARRIER_SUBSET, HF_BARRIER_BLOCKIDX = 0, 1, 2, 3
 HF_SPLIT_TABLE, HF_SPLIT_EXECTIME = -1, -2
 HF_MAX_SEARCH_RESULTS = 64
 HF_MAX_TENSORINFO_DIMS = 8
 
 ERROR_NAMES = {HF_EINVAL: "HF_EINVAL", HF_EPARSE: "HF_EPARSE", HF_ENOTFOUND: "HF_ENOTFOUND",
-               HF_EUNSUPPORTED: "HF_EUNSUPPORTED", HF_EHIP: "HF_EHIP", HF_EIO: "HF_EIO"}
+               HF_EUNSUPPORTED: "HF_EUNSUPPORTED", HF_EHIP: "HF_EHIP", HF_EIO: "HF_EIO", HF_ENOMEM: "HF_ENOMEM"}
 
 
 class HfuseError(RuntimeError):

@@ -8,6 +8,7 @@
 #include <fstream>
 #include <initializer_list>
 #include <mutex>
+#include <new>
 #include <sstream>
 #include <string>
 #include <vector>
@@ -32,6 +33,23 @@ int fail(int code, const std::string &msg) {
 
 int hip_fail(hipError_t e, const char *what) {
   return fail(HF_EHIP, std::string(what) + ": " + hipGetErrorString(e));
+}
+
+// No exception leaves the library: every entry point is a function-try-block that ends here.
+// (What can throw is host allocation: strings and vectors of the YAML model, plan objects.)
+int trap_exception() noexcept {
+  try {
+    throw;
+  } catch (const std::bad_alloc &) {
+    try { g_error.assign("out of memory"); } catch (...) {}   // fits the small-string buffer
+    return HF_ENOMEM;
+  } catch (const std::exception &e) {
+    try { g_error.assign(e.what()); } catch (...) {}
+    return HF_ENOMEM;
+  } catch (...) {
+    try { g_error.assign("unknown error"); } catch (...) {}
+    return HF_ENOMEM;
+  }
 }
 
 struct KernelName {
@@ -504,7 +522,7 @@ extern "C" {
 HF_API const char *hf_last_error(void) { return g_error.c_str(); }
 HF_API int hf_version(void) { return 100; }
 
-HF_API int hf_config_load_text(const char *fusion_yaml, const char *kernels_yaml, hf_config **out) {
+HF_API int hf_config_load_text(const char *fusion_yaml, const char *kernels_yaml, hf_config **out) try {
   if (!out) return fail(HF_EINVAL, "null output pointer");
   *out = nullptr;
   if (!kernels_yaml) return fail(HF_EINVAL, "null kernel table");
@@ -516,9 +534,11 @@ HF_API int hf_config_load_text(const char *fusion_yaml, const char *kernels_yaml
   }
   *out = c;
   return HF_OK;
+} catch (...) {
+  return trap_exception();
 }
 
-HF_API int hf_config_load_files(const char *fusion_path, const char *kernels_path, hf_config **out) {
+HF_API int hf_config_load_files(const char *fusion_path, const char *kernels_path, hf_config **out) try {
   if (!out) return fail(HF_EINVAL, "null output pointer");
   *out = nullptr;
   if (!kernels_path) return fail(HF_EINVAL, "null kernel table path");
@@ -534,6 +554,8 @@ HF_API int hf_config_load_files(const char *fusion_path, const char *kernels_pat
   if (!slurp(kernels_path, k)) return fail(HF_EIO, std::string("failed to read configs: ") + kernels_path);
   if (fusion_path && !slurp(fusion_path, f)) return fail(HF_EIO, std::string("failed to read configs: ") + fusion_path);
   return hf_config_load_text(fusion_path ? f.c_str() : nullptr, k.c_str(), out);
+} catch (...) {
+  return trap_exception();
 }
 
 HF_API void hf_config_free(hf_config *cfg) { delete cfg; }
@@ -541,7 +563,7 @@ HF_API void hf_config_free(hf_config *cfg) { delete cfg; }
 HF_API int hf_config_num_fusions(const hf_config *cfg) { return cfg ? (int)cfg->cfg.fusions.size() : fail(HF_EINVAL, "null config"); }
 HF_API int hf_config_num_kernels(const hf_config *cfg) { return cfg ? (int)cfg->cfg.rows.size() : fail(HF_EINVAL, "null config"); }
 
-HF_API int hf_config_fusion(const hf_config *cfg, int i, const char **file, const char **k1, const char **k2) {
+HF_API int hf_config_fusion(const hf_config *cfg, int i, const char **file, const char **k1, const char **k2) try {
   if (!cfg) return fail(HF_EINVAL, "null config");
   if (i < 0 || i >= (int)cfg->cfg.fusions.size()) return fail(HF_EINVAL, "fusion index out of range");
   const FusionRow &f = cfg->cfg.fusions[i];
@@ -549,9 +571,11 @@ HF_API int hf_config_fusion(const hf_config *cfg, int i, const char **file, cons
   if (k1) *k1 = f.kernels[0].c_str();
   if (k2) *k2 = f.kernels[1].c_str();
   return HF_OK;
+} catch (...) {
+  return trap_exception();
 }
 
-HF_API int hf_config_kernel(const hf_config *cfg, const char *name, hf_kernel_info *out) {
+HF_API int hf_config_kernel(const hf_config *cfg, const char *name, hf_kernel_info *out) try {
   if (!cfg || !name || !out) return fail(HF_EINVAL, "null argument");
   const KernelRow *r = cfg->cfg.find(name);
   if (!r) return fail(HF_ENOTFOUND, std::string("kernel '") + name + "' is not in the kernel table");
@@ -562,17 +586,21 @@ HF_API int hf_config_kernel(const hf_config *cfg, const char *name, hf_kernel_in
   out->reg = r->reg;
   out->exec_time = r->exec_time;
   return HF_OK;
+} catch (...) {
+  return trap_exception();
 }
 
-HF_API int hf_plan_num_splits(const hf_config *cfg, int fusion_index) {
+HF_API int hf_plan_num_splits(const hf_config *cfg, int fusion_index) try {
   if (!cfg) return fail(HF_EINVAL, "null config");
   if (fusion_index < 0 || fusion_index >= (int)cfg->cfg.fusions.size()) return fail(HF_EINVAL, "fusion index out of range");
   const FusionRow &f = cfg->cfg.fusions[fusion_index];
   return num_splits(*cfg->cfg.find(f.kernels[0]), *cfg->cfg.find(f.kernels[1]));
+} catch (...) {
+  return trap_exception();
 }
 
 HF_API int hf_plan_create(const hf_config *cfg, int fusion_index, const char *preset, int split_idx, int split_threads,
-                          hf_plan **out) {
+                          hf_plan **out) try {
   if (!out) return fail(HF_EINVAL, "null output pointer");
   *out = nullptr;
   if (!cfg || !preset) return fail(HF_EINVAL, "null argument");
@@ -636,9 +664,11 @@ HF_API int hf_plan_create(const hf_config *cfg, int fusion_index, const char *pr
   }
   *out = plan;
   return HF_OK;
+} catch (...) {
+  return trap_exception();
 }
 
-HF_API int hf_plan_set_barrier_mode(hf_plan *plan, int mode) {
+HF_API int hf_plan_set_barrier_mode(hf_plan *plan, int mode) try {
   if (!plan) return fail(HF_EINVAL, "null plan");
   const bool b1 = body_has_barriers(plan->ids[0]), b2 = body_has_barriers(plan->ids[1]);
   switch (mode) {
@@ -658,17 +688,21 @@ HF_API int hf_plan_set_barrier_mode(hf_plan *plan, int mode) {
   }
   plan->barrier_mode = mode;
   return HF_OK;
+} catch (...) {
+  return trap_exception();
 }
 
-HF_API int hf_plan_set_grids(hf_plan *plan, int grid1, int grid2) {
+HF_API int hf_plan_set_grids(hf_plan *plan, int grid1, int grid2) try {
   if (!plan) return fail(HF_EINVAL, "null plan");
   if (grid1 < 0 || grid2 < 0) return fail(HF_EINVAL, "negative grid");
   plan->grid_override[0] = (unsigned)grid1;
   plan->grid_override[1] = (unsigned)grid2;
   return HF_OK;
+} catch (...) {
+  return trap_exception();
 }
 
-HF_API int hf_plan_set_block(hf_plan *plan, int threads1, int threads2) {
+HF_API int hf_plan_set_block(hf_plan *plan, int threads1, int threads2) try {
   if (!plan) return fail(HF_EINVAL, "null plan");
   if (plan->preset->base_line) return fail(HF_EINVAL, "vertical presets have no thread partition to set");
   if (threads1 <= 0 || threads2 <= 0 || threads1 % (int)kWave || threads2 % (int)kWave)
@@ -691,23 +725,29 @@ HF_API int hf_plan_set_block(hf_plan *plan, int threads1, int threads2) {
               std::to_string(threads1) + "_" + std::to_string(threads2);
   plan->part = part;
   return HF_OK;
+} catch (...) {
+  return trap_exception();
 }
 
-HF_API int hf_plan_set_lending(hf_plan *plan, int on) {
+HF_API int hf_plan_set_lending(hf_plan *plan, int on) try {
   if (!plan) return fail(HF_EINVAL, "null plan");
   plan->lending = on != 0;
   return HF_OK;
+} catch (...) {
+  return trap_exception();
 }
 
-HF_API int hf_plan_set_launch_bound(hf_plan *plan, int on) {
+HF_API int hf_plan_set_launch_bound(hf_plan *plan, int on) try {
   if (!plan) return fail(HF_EINVAL, "null plan");
   plan->bounded = on < 0 ? -1 : (on != 0);
   return HF_OK;
+} catch (...) {
+  return trap_exception();
 }
 
 HF_API void hf_plan_free(hf_plan *plan) { delete plan; }
 
-HF_API int hf_plan_partition(const hf_plan *plan, hf_partition *out) {
+HF_API int hf_plan_partition(const hf_plan *plan, hf_partition *out) try {
   if (!plan || !out) return fail(HF_EINVAL, "null argument");
   std::memset(out, 0, sizeof *out);
   std::strncpy(out->name, plan->part.name.c_str(), sizeof out->name - 1);
@@ -720,9 +760,11 @@ HF_API int hf_plan_partition(const hf_plan *plan, hf_partition *out) {
   out->launch_blocks = plan->part.launch_blocks;
   out->barrier_mode = plan->barrier_mode;
   return HF_OK;
+} catch (...) {
+  return trap_exception();
 }
 
-HF_API int hf_plan_local_index(const hf_plan *plan, int half, uint32_t tid, hf_dim3 *out) {
+HF_API int hf_plan_local_index(const hf_plan *plan, int half, uint32_t tid, hf_dim3 *out) try {
   if (!plan || !out) return fail(HF_EINVAL, "null argument");
   if (half < 0 || half > 1) return fail(HF_EINVAL, "half must be 0 or 1");
   if (tid < plan->part.lo[half] || tid >= plan->part.hi[half])
@@ -730,11 +772,13 @@ HF_API int hf_plan_local_index(const hf_plan *plan, int half, uint32_t tid, hf_d
   Dim3 d = local_index(tid, plan->part.lo[half], plan->part.block_dim[half]);
   *out = {d.x, d.y, d.z};
   return HF_OK;
+} catch (...) {
+  return trap_exception();
 }
 
 // ------------------------------------------------------------- constants
 HF_API int hf_ethash_set_constants(const void *dag, uint32_t dag_items, const uint8_t header[32], uint64_t target,
-                                   void *) {
+                                   void *) try {
   if (!dag || !header) return fail(HF_EINVAL, "ethash: null dag or header");
   if (dag_items == 0) return fail(HF_EINVAL, "ethash: empty dag");
   if (!aligned16(dag)) return fail(HF_EINVAL, "ethash: dag must be 16-byte aligned");
@@ -745,9 +789,11 @@ HF_API int hf_ethash_set_constants(const void *dag, uint32_t dag_items, const ui
   g_const.eth_target = target;
   g_const.eth_set = true;
   return HF_OK;
+} catch (...) {
+  return trap_exception();
 }
 
-HF_API int hf_sha256d_set_block(const uint8_t header[80], uint64_t target64, void *) {
+HF_API int hf_sha256d_set_block(const uint8_t header[80], uint64_t target64, void *) try {
   if (!header) return fail(HF_EINVAL, "sha256d: null header");
   uint32_t st[8] = {0x6a09e667, 0xbb67ae85, 0x3c6ef372, 0xa54ff53a, 0x510e527f, 0x9b05688c, 0x1f83d9ab, 0x5be0cd19};
   uint32_t blk[16];
@@ -759,27 +805,33 @@ HF_API int hf_sha256d_set_block(const uint8_t header[80], uint64_t target64, voi
   g_const.sha_target = target64;
   g_const.sha_set = true;
   return HF_OK;
+} catch (...) {
+  return trap_exception();
 }
 
-HF_API int hf_sia_blake2b_set_block(const uint8_t header[80], void *) {
+HF_API int hf_sia_blake2b_set_block(const uint8_t header[80], void *) try {
   if (!header) return fail(HF_EINVAL, "sia_blake2b: null header");
   std::lock_guard<std::mutex> lock(g_const.mu);
   for (int i = 0; i < 10; i++) g_const.sia_m[i] = load_le64(header + 8 * i);
   g_const.sia_set = true;
   return HF_OK;
+} catch (...) {
+  return trap_exception();
 }
 
-HF_API int hf_blake2b_set_block(const uint8_t header[80], void *) {
+HF_API int hf_blake2b_set_block(const uint8_t header[80], void *) try {
   if (!header) return fail(HF_EINVAL, "blake2b: null header");
   std::lock_guard<std::mutex> lock(g_const.mu);
   for (int i = 0; i < 10; i++) g_const.b2_m[i] = load_le64(header + 8 * i);
   g_const.b2_set = true;
   return HF_OK;
+} catch (...) {
+  return trap_exception();
 }
 
 // ---------------------------------------------------------------- launches
 HF_API int hf_launch_native(const char *kernel_name, const void *args, int grid_blocks, int block_threads,
-                            void *stream) {
+                            void *stream) try {
   if (!kernel_name) return fail(HF_EINVAL, "null kernel name");
   KernelId id;
   if (!lookup_kernel(kernel_name, id))
@@ -789,6 +841,8 @@ HF_API int hf_launch_native(const char *kernel_name, const void *args, int grid_
   if (rc != HF_OK) return rc;
   unsigned block = block_threads > 0 ? (unsigned)block_threads : (is_crypto(id) ? 128u : (id == K_MAXPOOL ? 256u : 512u));
   return do_launch_native(id, p, grid_blocks, block, static_cast<hipStream_t>(stream));
+} catch (...) {
+  return trap_exception();
 }
 
 namespace {
@@ -872,7 +926,7 @@ int do_launch_fused(const hf_plan *plan, const Prepared &p1, const Prepared &p2,
 
 }  // namespace
 
-HF_API int hf_launch_fused(const hf_plan *plan, const void *args1, const void *args2, int grid_blocks, void *stream) {
+HF_API int hf_launch_fused(const hf_plan *plan, const void *args1, const void *args2, int grid_blocks, void *stream) try {
   if (!plan) return fail(HF_EINVAL, "null plan");
   Prepared p1, p2;
   int rc = prepare(plan->ids[0], args1, p1);
@@ -880,10 +934,12 @@ HF_API int hf_launch_fused(const hf_plan *plan, const void *args1, const void *a
   rc = prepare(plan->ids[1], args2, p2);
   if (rc != HF_OK) return rc;
   return do_launch_fused(plan, p1, p2, grid_blocks, static_cast<hipStream_t>(stream));
+} catch (...) {
+  return trap_exception();
 }
 
 HF_API int hf_time_pair(const hf_plan *plan, int mode, const void *const *args1, const void *const *args2, int nsets,
-                        int warmup, int iters, int grid_blocks, void *stream_, float *elapsed_ms) {
+                        int warmup, int iters, int grid_blocks, void *stream_, float *elapsed_ms) try {
   if (!plan || !args1 || !args2 || !elapsed_ms) return fail(HF_EINVAL, "null argument");
   if (nsets <= 0 || iters <= 0 || warmup < 0 || mode < 0 || mode > 4) return fail(HF_EINVAL, "bad repetition arguments");
   hipStream_t stream = static_cast<hipStream_t>(stream_);
@@ -959,20 +1015,26 @@ HF_API int hf_time_pair(const hf_plan *plan, int mode, const void *const *args1,
   if (rc != HF_OK) return rc;
   if (e != hipSuccess) return hip_fail(e, "timing");
   return HF_OK;
+} catch (...) {
+  return trap_exception();
 }
 
-HF_API int hf_fill_splitmix64(uint64_t *dst, uint64_t nwords, uint64_t seed, void *stream) {
+HF_API int hf_fill_splitmix64(uint64_t *dst, uint64_t nwords, uint64_t seed, void *stream) try {
   if (!dst && nwords) return fail(HF_EINVAL, "null destination");
   hipError_t e = launch_fill_splitmix64(reinterpret_cast<unsigned long long *>(dst), nwords, seed, static_cast<hipStream_t>(stream));
   if (e != hipSuccess) return hip_fail(e, "fill launch");
   return HF_OK;
+} catch (...) {
+  return trap_exception();
 }
 
-HF_API int hf_copy_f32(const float *src, float *dst, uint64_t n, void *stream) {
+HF_API int hf_copy_f32(const float *src, float *dst, uint64_t n, void *stream) try {
   if ((!src || !dst) && n) return fail(HF_EINVAL, "null pointer");
   hipError_t e = launch_copy_f32(src, dst, n, static_cast<hipStream_t>(stream));
   if (e != hipSuccess) return hip_fail(e, "copy launch");
   return HF_OK;
+} catch (...) {
+  return trap_exception();
 }
 
 }  // extern "C"

@@ -1,6 +1,5 @@
 #include "yaml_lite.h"
 
-#include <sstream>
 
 namespace hfuse {
 namespace {
@@ -57,9 +56,7 @@ struct Parser {
   std::string err;
 
   bool fail(int no, const std::string &why) {
-    std::ostringstream o;
-    o << "line " << no << ": " << why;
-    err = o.str();
+    err = "line " + std::to_string(no) + ": " + why;
     return false;
   }
 
@@ -145,16 +142,19 @@ struct Parser {
 
 bool yaml_parse(const std::string &text, YamlNode &root, std::string &err) {
   Parser p;
-  std::istringstream in(text);
+  // Lines are cut by hand: a stream would swallow an allocation failure inside getline and
+  // merely look exhausted, which turns "out of memory" into a parse error about a short file.
   std::string raw;
   int no = 0;
-  while (std::getline(in, raw)) {
+  for (size_t at = 0; at < text.size();) {
+    const size_t nl = text.find('\n', at);
+    const size_t end = nl == std::string::npos ? text.size() : nl;
+    raw.assign(text, at, end - at);
+    at = end + 1;
     no++;
     if (raw.find('\t') != std::string::npos && raw.find_first_not_of(" \t") != std::string::npos &&
         raw.substr(0, raw.find_first_not_of(" \t")).find('\t') != std::string::npos) {
-      std::ostringstream o;
-      o << "line " << no << ": tab in indentation";
-      err = o.str();
+      err = "line " + std::to_string(no) + ": tab in indentation";
       return false;
     }
     std::string s = rstrip(strip_comment(raw));
@@ -170,9 +170,7 @@ bool yaml_parse(const std::string &text, YamlNode &root, std::string &err) {
     return false;
   }
   if (p.pos != p.lines.size()) {
-    std::ostringstream o;
-    o << "line " << p.lines[p.pos].no << ": inconsistent indentation";
-    err = o.str();
+    err = "line " + std::to_string(p.lines[p.pos].no) + ": inconsistent indentation";
     return false;
   }
   return true;

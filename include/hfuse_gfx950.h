@@ -47,7 +47,8 @@ enum {
   HF_ENOTFOUND = -3,   /* unknown kernel / pair / preset                       */
   HF_EUNSUPPORTED = -4,/* legal in the reference, not built here               */
   HF_EHIP = -5,        /* a HIP runtime call failed                            */
-  HF_EIO = -6          /* file could not be read                               */
+  HF_EIO = -6,         /* file could not be read                               */
+  HF_ENOMEM = -7       /* host allocation failed (or another C++ exception)    */
 };
 
 HF_API const char *hf_last_error(void);

@@ -42,3 +42,18 @@ def test_block_dim_must_be_launchable(dim):
     with pytest.raises(hfuse_amd.HfuseError) as e:
         Config("- File: a\n  Kernels:\n    - k\n    - k\n", table)
     assert e.value.code == L.HF_EPARSE and "BlockDim" in e.value.message
+
+
+def test_allocation_failures_come_back_as_error_codes(tmp_path):
+    """Every host allocation of config loading and plan creation fails once (injected through a
+    replaced `operator new`): the C-ABI answers HF_ENOMEM, no exception crosses the boundary."""
+    exe = str(tmp_path / "alloc_fault")
+    subprocess.check_call(["g++", "-std=c++17", "-O1", "-g", "-I", os.path.join(HERE, "..", "include"),
+                           os.path.join(HERE, "alloc_fault.cpp"), "-L", PKG, "-lhfuse_gfx950",
+                           "-Wl,-rpath," + PKG, "-o", exe])
+    r = subprocess.run([exe, os.path.join(PKG, "configs", "gfx950_fusion.yaml"),
+                        os.path.join(PKG, "configs", "gfx950_kernels.yaml")],
+                       capture_output=True, text=True, timeout=300)
+    assert r.returncode == 0, (r.stdout + r.stderr)[-2000:]
+    words = r.stdout.split()
+    assert int(words[1]) > 100 and int(words[3]) >= 1   # that many distinct allocations were failed
