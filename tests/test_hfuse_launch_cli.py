@@ -22,7 +22,8 @@ def run(*extra):
 def test_every_shipped_pair_small(cuda):
     cfg = hfuse_amd.default_config()
     for i, (file, k1, k2) in enumerate(cfg.fusions()):
-        for extra in ((), ("--preset", "vfuse")) if i < 5 else ((),):
+        # the benchmarked pairs also under the vertical and the register-bounded presets
+        for extra in ((), ("--preset", "vfuse"), ("--preset", "hfuse_lb"), ("--preset", "vfuse_lb")) if i < 5 else ((),):
             r = run(str(i), "--small", "--iters", "3", *extra)
             assert r.returncode == 0, (file, r.stdout, r.stderr)
             assert f"fused == native: {k1} yes, {k2} yes" in r.stdout
