@@ -51,6 +51,9 @@ def parse():
     ap.add_argument("--search-log2", type=int, default=None, help="override log2 of the nonce ranges (debug)")
     ap.add_argument("--extra-pairs", action="store_true",
                     help="also time the other tensor pairs of the shipped fusion list (the reference's ml_fusion.yaml)")
+    ap.add_argument("--read-footprint-mb", type=int, default=0,
+                    help="MB the smaller read stream of a tensor pair cycles through before a buffer set repeats "
+                         "(default 600: several GB of buffers in rotation; at least three sets in any case)")
     ap.add_argument("--calibrate-copy", type=int, default=0, metavar="MIB",
                     help="also run the plain copy kernel on MIB mebibytes (the unit HBM counters are scaled by)")
     return ap.parse_args()
@@ -290,6 +293,9 @@ def cpu_baseline_search(name, seconds=6.0):
 # ------------------------------------------------------------------ main
 def main():
     args = parse()
+    if args.read_footprint_mb > 0:
+        import hfuse_amd.workloads as workloads
+        workloads.MIN_READ_FOOTPRINT = args.read_footprint_mb << 20
     if args.gpus != 1:
         print("bench.py: this build runs on one GPU only (every pair would shard without an exchange step); "
               "--gpus must be 1", file=sys.stderr)

@@ -15,17 +15,25 @@ TENSOR_KERNELS = ("im2col_kernel", "MaxPoolForward", "batch_norm_collect_statist
 SEARCH_KERNELS = ("ethash_search", "sha256d_gpu_hash_shared", "sia_blake2b_gpu_hash", "blake2b_gpu_hash")
 
 
+# Bytes the smaller read stream of a pair cycles through before a buffer set repeats.  The default
+# puts several GB between two uses of a buffer: no cache and no translation entry survives that.
+MIN_READ_FOOTPRINT = 600 << 20
+
+
 class TensorPair:
     """One tensor pair: `nsets` independent input/output sets so repeats miss the last-level cache."""
 
-    def __init__(self, name, k1, k2, make_set, bytes1, bytes2, min_read_footprint=600 << 20):
+    def __init__(self, name, k1, k2, make_set, bytes1, bytes2, min_read_footprint=None):
         # Enough sets that even the smaller of the two read streams cycles through more bytes
         # than the 256 MB memory-side cache holds, so neither kernel re-reads cached inputs.
+        # (At least three sets whatever the footprint asked for.)
+        if min_read_footprint is None:
+            min_read_footprint = MIN_READ_FOOTPRINT
         self.name, self.k1, self.k2 = name, k1, k2
         self.bytes1, self.bytes2 = bytes1, bytes2
         self.sets = []
         read_footprint = 0
-        while read_footprint < min_read_footprint or len(self.sets) < 2:
+        while read_footprint < min_read_footprint or len(self.sets) < 3:
             s = make_set(len(self.sets))
             self.sets.append(s)
             read_footprint += s["min_read"]
