@@ -53,7 +53,7 @@ def parse():
                     help="also time the other tensor pairs of the shipped fusion list (the reference's ml_fusion.yaml)")
     ap.add_argument("--read-footprint-mb", type=int, default=0,
                     help="MB the smaller read stream of a tensor pair cycles through before a buffer set repeats "
-                         "(default 600: several GB of buffers in rotation; at least three sets in any case)")
+                         "(default 600; below about 300 the memory-side cache serves the reads; at least three sets in any case)")
     ap.add_argument("--calibrate-copy", type=int, default=0, metavar="MIB",
                     help="also run the plain copy kernel on MIB mebibytes (the unit HBM counters are scaled by)")
     return ap.parse_args()

@@ -15,8 +15,9 @@ TENSOR_KERNELS = ("im2col_kernel", "MaxPoolForward", "batch_norm_collect_statist
 SEARCH_KERNELS = ("ethash_search", "sha256d_gpu_hash_shared", "sia_blake2b_gpu_hash", "blake2b_gpu_hash")
 
 
-# Bytes the smaller read stream of a pair cycles through before a buffer set repeats.  The default
-# puts several GB between two uses of a buffer: no cache and no translation entry survives that.
+# Bytes the smaller read stream of a pair cycles through before a buffer set repeats.  It is the
+# inputs alone that have to outgrow the 256 MB memory-side cache: the outputs are written with
+# non-temporal stores and take no room there, so ten sets of a 25 MB input still read from cache.
 MIN_READ_FOOTPRINT = 600 << 20
 
 
