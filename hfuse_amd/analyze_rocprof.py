@@ -193,7 +193,10 @@ def derived_metrics(c: Dict[str, float], cus: int = 256, xcds: int = 8) -> Dict[
       mem_stalled_pct (stall_memory_dependency)  rocprofv3's own derived MemUnitStalled, when collected
       wait_issue_pct  (no nvprof counterpart)    100 * SQ_WAIT_INST_ANY / SQ_WAVE_CYCLES: wave-cycles spent
                       waiting for an earlier instruction of any kind, other waves' turns on the SIMD included
-      occupancy_pct   (achieved_occupancy)       100 * 4 * SQ_WAVE_CYCLES / busy / CUs / 32 wave slots"""
+      occupancy_pct   (achieved_occupancy)       100 * 4 * SQ_WAVE_CYCLES / busy / CUs / 32 wave slots
+      lds_busy_pct    (no nvprof counterpart)    100 * SQ_LDS_IDX_ACTIVE / CUs / busy (rocprofv3's LdsUtil)
+      lds_conflict_pct                           100 * SQ_LDS_BANK_CONFLICT / SQ_LDS_IDX_ACTIVE: share of the
+                      LDS's active cycles lost to bank conflicts (the histogram's atomics on random bins)"""
     out: Dict[str, float] = {}
     busy = c.get("GRBM_GUI_ACTIVE", 0.0) / xcds
     if busy > 0 and "SQ_ACTIVE_INST_VALU" in c:
@@ -204,6 +207,12 @@ def derived_metrics(c: Dict[str, float], cus: int = 256, xcds: int = 8) -> Dict[
         out["wait_issue_pct"] = 100.0 * c["SQ_WAIT_INST_ANY"] / c["SQ_WAVE_CYCLES"]
     if "MemUnitStalled" in c:
         out["mem_stalled_pct"] = c["MemUnitStalled"]
+    if busy > 0 and "SQ_LDS_IDX_ACTIVE" in c:
+        out["lds_busy_pct"] = 100.0 * c["SQ_LDS_IDX_ACTIVE"] / cus / busy
+    if c.get("SQ_LDS_IDX_ACTIVE", 0.0) > 0 and "SQ_LDS_BANK_CONFLICT" in c:
+        out["lds_conflict_pct"] = 100.0 * c["SQ_LDS_BANK_CONFLICT"] / c["SQ_LDS_IDX_ACTIVE"]
+    if "SQ_INSTS_LDS" in c:
+        out["lds_insts"] = c["SQ_INSTS_LDS"]
     if "SQ_WAVES" in c:
         out["waves"] = c["SQ_WAVES"]
     if "SQ_INSTS_VALU" in c:
@@ -261,7 +270,9 @@ def render_exec_table(table, fmt: str = "md") -> str:
 
 _METRIC_COLS = (("valu_busy_pct", "VALU busy %", "{:.1f}"), ("mem_stalled_pct", "mem unit stalled %", "{:.1f}"),
                 ("wait_issue_pct", "waiting on issue %", "{:.1f}"),
-                ("occupancy_pct", "occupancy %", "{:.1f}"), ("waves", "waves", "{:.0f}"),
+                ("occupancy_pct", "occupancy %", "{:.1f}"), ("lds_busy_pct", "LDS busy %", "{:.1f}"),
+                ("lds_conflict_pct", "LDS bank conflicts % of LDS cycles", "{:.1f}"), ("lds_insts", "LDS insts", "{:.0f}"),
+                ("waves", "waves", "{:.0f}"),
                 ("valu_insts", "VALU insts", "{:.0f}"), ("fetch_kib", "FETCH_SIZE KiB", "{:.1f}"),
                 ("write_kib", "WRITE_SIZE KiB", "{:.1f}"))
 

@@ -110,3 +110,10 @@ def test_metric_table(tmp_path):
                     "Counter_Name": "SQ_WAVES", "Counter_Value": 16.0})
     labels = [(n, t) for n, t, _ in A.metric_table(A.load_counters([str(p)]))]
     assert labels == [("SHA256", "ST grid 1024"), ("SHA256", "ST grid 1048576"), ("SHA256+Blake2B", "HF@256")]
+
+
+def test_lds_metrics():
+    m = A.derived_metrics({"GRBM_GUI_ACTIVE": 8 * 1000.0, "SQ_LDS_IDX_ACTIVE": 256 * 250.0, "SQ_LDS_BANK_CONFLICT": 256 * 100.0,
+                           "SQ_INSTS_LDS": 4096.0})
+    assert m["lds_busy_pct"] == pytest.approx(25.0) and m["lds_conflict_pct"] == pytest.approx(40.0) and m["lds_insts"] == 4096.0
+    assert "lds_busy_pct" not in A.derived_metrics({"GRBM_GUI_ACTIVE": 8000.0})
