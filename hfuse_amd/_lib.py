@@ -130,6 +130,8 @@ PROTOTYPES = {
     "hf_config_num_kernels": (C.c_int, [C.c_void_p]),
     "hf_config_fusion": (C.c_int, [C.c_void_p, C.c_int, C.POINTER(C.c_char_p), C.POINTER(C.c_char_p),
                                    C.POINTER(C.c_char_p)]),
+    "hf_config_fusion_size": (C.c_int, [C.c_void_p, C.c_int]),
+    "hf_config_fusion_kernel": (C.c_int, [C.c_void_p, C.c_int, C.c_int, C.POINTER(C.c_char_p)]),
     "hf_config_kernel": (C.c_int, [C.c_void_p, C.c_char_p, C.POINTER(KernelInfo)]),
     "hf_plan_create": (C.c_int, [C.c_void_p, C.c_int, C.c_char_p, C.c_int, C.c_int, C.POINTER(C.c_void_p)]),
     "hf_plan_free": (None, [C.c_void_p]),

@@ -516,6 +516,15 @@ struct hf_plan {
   int bounded = -1;                    // hf_plan_set_launch_bound: 0 / 1, -1 = by the preset
 };
 
+namespace {
+// The reference's Context partitions a block among any number of kernels (include/KernelFusion.h:45-80;
+// configs/crypt_four.yaml fuses three); fused kernels are built for pairs here.
+int pairs_only(const FusionRow &f) {
+  return fail(HF_EUNSUPPORTED, "fusion '" + f.file + "' names " + std::to_string(f.kernels.size()) +
+                                   " kernels: fused kernels are built for pairs");
+}
+}  // namespace
+
 // ------------------------------------------------------------------ C-ABI
 extern "C" {
 
@@ -569,10 +578,25 @@ HF_API int hf_config_fusion(const hf_config *cfg, int i, const char **file, cons
   const FusionRow &f = cfg->cfg.fusions[i];
   if (file) *file = f.file.c_str();
   if (k1) *k1 = f.kernels[0].c_str();
-  if (k2) *k2 = f.kernels[1].c_str();
+  if (k2) *k2 = f.kernels.size() > 1 ? f.kernels[1].c_str() : "";
   return HF_OK;
 } catch (...) {
   return trap_exception();
+}
+
+HF_API int hf_config_fusion_size(const hf_config *cfg, int i) {
+  if (!cfg) return fail(HF_EINVAL, "null config");
+  if (i < 0 || i >= (int)cfg->cfg.fusions.size()) return fail(HF_EINVAL, "fusion index out of range");
+  return (int)cfg->cfg.fusions[i].kernels.size();
+}
+
+HF_API int hf_config_fusion_kernel(const hf_config *cfg, int i, int k, const char **name) {
+  if (!cfg || !name) return fail(HF_EINVAL, "null argument");
+  if (i < 0 || i >= (int)cfg->cfg.fusions.size()) return fail(HF_EINVAL, "fusion index out of range");
+  const FusionRow &f = cfg->cfg.fusions[i];
+  if (k < 0 || k >= (int)f.kernels.size()) return fail(HF_EINVAL, "kernel index out of range");
+  *name = f.kernels[k].c_str();
+  return HF_OK;
 }
 
 HF_API int hf_config_kernel(const hf_config *cfg, const char *name, hf_kernel_info *out) try {
@@ -594,6 +618,7 @@ HF_API int hf_plan_num_splits(const hf_config *cfg, int fusion_index) try {
   if (!cfg) return fail(HF_EINVAL, "null config");
   if (fusion_index < 0 || fusion_index >= (int)cfg->cfg.fusions.size()) return fail(HF_EINVAL, "fusion index out of range");
   const FusionRow &f = cfg->cfg.fusions[fusion_index];
+  if (f.kernels.size() != 2) return pairs_only(f);
   return num_splits(*cfg->cfg.find(f.kernels[0]), *cfg->cfg.find(f.kernels[1]));
 } catch (...) {
   return trap_exception();
@@ -610,6 +635,7 @@ HF_API int hf_plan_create(const hf_config *cfg, int fusion_index, const char *pr
   if (split_threads > 0 && split_threads % (int)kWave != 0)
     return fail(HF_EINVAL, "split_threads must be a multiple of the 64-lane wavefront");
   const FusionRow &f = cfg->cfg.fusions[fusion_index];
+  if (f.kernels.size() != 2) return pairs_only(f);
   auto plan = new hf_plan();
   plan->preset = p;
   for (int i = 0; i < 2; i++) {

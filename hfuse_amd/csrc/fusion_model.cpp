@@ -194,7 +194,8 @@ bool parse_config(const char *fusion_yaml, const char *kernels_yaml, Config &cfg
     }
   }
   for (auto &f : cfg.fusions) {
-    if (f.kernels.size() != 2) { err = "fusion '" + f.file + "': exactly two kernels are fused"; return false; }
+    // (the schema allows any number of kernels, include/KernelFusion.h:140-146; plans are built for pairs)
+    if (f.kernels.empty()) { err = "fusion '" + f.file + "': no kernels"; return false; }
     for (auto &k : f.kernels)
       if (!cfg.find(k)) { err = "fusion '" + f.file + "': kernel '" + k + "' is not in the kernel table"; return false; }
   }

@@ -60,9 +60,19 @@ class Config:
     def fusions(self):
         return [self.fusion(i) for i in range(self.num_fusions)]
 
+    def fusion_kernels(self, i: int):
+        """All kernel names of entry i (the schema allows any number; plans exist for pairs)."""
+        n = check(L.lib().hf_config_fusion_size(self._h, i))
+        out = []
+        for k in range(n):
+            name = C.c_char_p()
+            check(L.lib().hf_config_fusion_kernel(self._h, i, k, C.byref(name)))
+            out.append(name.value.decode())
+        return out
+
     def find_fusion(self, k1: str, k2: str) -> int:
         for i, (_, a, b) in enumerate(self.fusions()):
-            if (a, b) == (k1, k2):
+            if (a, b) == (k1, k2) and check(L.lib().hf_config_fusion_size(self._h, i)) == 2:
                 return i
         raise KeyError(f"no fusion of {k1} + {k2} in the fusion list")
 

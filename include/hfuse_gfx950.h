@@ -90,9 +90,17 @@ HF_API int hf_config_load_files(const char *fusion_path, const char *kernels_pat
 HF_API void hf_config_free(hf_config *cfg);
 HF_API int hf_config_num_fusions(const hf_config *cfg);
 HF_API int hf_config_num_kernels(const hf_config *cfg);
-/* Names of the i-th fusion's kernels (NUL-terminated, valid while cfg lives). */
+/*
+ * Names of the i-th fusion's kernels (NUL-terminated, valid while cfg lives).  The schema lets an
+ * entry name any number of kernels (include/KernelFusion.h:140-146; configs/crypt_four.yaml names
+ * three): such a list loads, hf_config_fusion gives its first two names (k2 = "" for a single one),
+ * hf_config_fusion_size / hf_config_fusion_kernel give all of them, and hf_plan_create answers
+ * HF_EUNSUPPORTED for every entry that is not a pair.
+ */
 HF_API int hf_config_fusion(const hf_config *cfg, int i, const char **file, const char **k1,
                             const char **k2);
+HF_API int hf_config_fusion_size(const hf_config *cfg, int i);
+HF_API int hf_config_fusion_kernel(const hf_config *cfg, int i, int k, const char **name);
 HF_API int hf_config_kernel(const hf_config *cfg, const char *name, hf_kernel_info *out);
 
 /* ------------------------------------------------------------------- plans */

@@ -119,9 +119,26 @@ def test_fusion_list_errors():
     with pytest.raises(hfuse_amd.HfuseError) as e:
         Config("- File: f\n  Kernels:\n    - im2col_kernel\n    - nope\n", KERNELS_MAP)
     assert e.value.code == L.HF_EPARSE and "nope" in e.value.message
+    # the schema allows any number of kernels per entry (the reference's crypt_four.yaml names three):
+    # such a list loads, and only asking for a plan of a non-pair is refused
+    cfg = Config("- File: one\n  Kernels:\n    - im2col_kernel\n"
+                 "- File: three\n  Kernels:\n    - im2col_kernel\n    - MaxPoolForward\n    - im2col_kernel\n"
+                 "- File: two\n  Kernels:\n    - im2col_kernel\n    - MaxPoolForward\n", KERNELS_MAP)
+    assert cfg.num_fusions == 3
+    assert cfg.fusion(0) == ("one", "im2col_kernel", "")
+    assert cfg.fusion_kernels(1) == ["im2col_kernel", "MaxPoolForward", "im2col_kernel"]
+    assert cfg.find_fusion("im2col_kernel", "MaxPoolForward") == 2      # the triple is not mistaken for the pair
+    for i in (0, 1):
+        with pytest.raises(hfuse_amd.HfuseError) as e:
+            cfg.plan(i)
+        assert e.value.code == L.HF_EUNSUPPORTED and "pairs" in e.value.message
+        with pytest.raises(hfuse_amd.HfuseError) as e:
+            cfg.num_splits(i)
+        assert e.value.code == L.HF_EUNSUPPORTED
+    cfg.plan(2)
     with pytest.raises(hfuse_amd.HfuseError) as e:
-        Config("- File: f\n  Kernels:\n    - im2col_kernel\n", KERNELS_MAP)
-    assert "exactly two" in e.value.message
+        Config("- File: f\n  Kernels: []\n", KERNELS_MAP)
+    assert e.value.code == L.HF_EPARSE
     with pytest.raises(hfuse_amd.HfuseError) as e:
         Config("- Kernels:\n    - im2col_kernel\n    - MaxPoolForward\n", KERNELS_MAP)
     assert "File" in e.value.message
