@@ -5,7 +5,7 @@
 // prints the per-launch durations, and checks that the fused launch produced the same bytes
 // as the two native launches (batch-norm statistics: the same values to 1e-5 relative).
 //
-//   hfuse-launch <fusion.yaml> <kernels.yaml> <File name | index> [--preset P] [--split N]
+//   hfuse-launch <fusion.yaml> <kernels.yaml> <File name | index | all> [--preset P] [--split N]
 //                [--iters N] [--small]
 //
 // Inputs are the benchmark shapes (--small: shapes a thousand times smaller), filled from
@@ -254,11 +254,57 @@ bool same_outputs(const Workload &w) {
   return true;
 }
 
+// One pair: a compared launch of each form on identical inputs, then timed repetitions.
+// Returns the speedup of the fused kernel over back to back in percent; `ok` = outputs agree.
+double run_pair(hf_config *cfg, int index, const std::string &preset, int split, int iters, bool small, bool &ok) {
+  const char *file = "", *k1 = "", *k2 = "";
+  hf_check(hf_config_fusion(cfg, index, &file, &k1, &k2));
+  hf_plan *plan = nullptr;
+  hf_check(hf_plan_create(cfg, index, preset.c_str(), split, 0, &plan));
+  hf_partition part;
+  hf_check(hf_plan_partition(plan, &part));
+  std::printf("%s: %s + %s as %s (%u threads: [%u,%u) + [%u,%u))\n", file, k1, k2, part.name, part.launch_threads,
+              part.lo[0], part.hi[0], part.lo[1], part.hi[1]);
+
+  const bool hist_pair = std::string(k1) == "kernelHistogram1D";
+  auto w1 = make_workload(k1, false, small, 0x48467573ull);
+  auto w2 = make_workload(k2, hist_pair, small, 0x48467574ull);
+  // ethash scans grid * (its block) nonces: natively 128-thread blocks, fused its share of the block
+  const int native_grid = w1->grid ? w1->grid : w2->grid;
+  int fused_grid = 0;
+  if (w1->grid) fused_grid = (int)(w1->hashes / (part.hi[0] - part.lo[0]));
+  if (w2->grid) fused_grid = (int)(w2->hashes / (part.hi[1] - part.lo[1]));
+
+  w1->reset();
+  w2->reset();
+  hip_check(hipDeviceSynchronize(), "reset");
+  hf_check(hf_launch_native(k1, w1->args_native.data(), w1->grid, 0, nullptr));
+  hf_check(hf_launch_native(k2, w2->args_native.data(), w2->grid, 0, nullptr));
+  hf_check(hf_launch_fused(plan, w1->args_fused.data(), w2->args_fused.data(), fused_grid, nullptr));
+  hip_check(hipDeviceSynchronize(), "compared launches");
+  const bool ok1 = same_outputs(*w1), ok2 = same_outputs(*w2);
+  std::printf("fused == native: %s %s, %s %s\n", k1, ok1 ? "yes" : "NO", k2, ok2 ? "yes" : "NO");  // batch-norm: to 1e-5 relative
+
+  // timed repetitions: A, B, A then B, fused
+  const void *a1[1] = {w1->args_native.data()}, *a2[1] = {w2->args_native.data()};
+  const char *label[4] = {k1, k2, "back to back", part.name};
+  float ms[4];
+  for (int mode = 0; mode < 4; mode++) {
+    hf_check(hf_time_pair(plan, mode, a1, a2, 1, 2, iters, mode == 3 ? fused_grid : native_grid, nullptr, &ms[mode]));
+    std::printf("%-60s %10.3f us per launch\n", label[mode], 1e3 * ms[mode] / iters);
+  }
+  const double speedup = (ms[2] / ms[3] - 1.0) * 100.0;
+  std::printf("speedup of the fused kernel over back to back: %+.1f %%\n", speedup);
+  hf_plan_free(plan);
+  ok = ok1 && ok2;
+  return speedup;
+}
+
 }  // namespace
 
 int main(int argc, char **argv) {
   if (argc < 4) {
-    std::fprintf(stderr, "usage: %s <fusion.yaml> <kernels.yaml> <File name | index> [--preset P] [--split N] [--iters N] [--small]\n", argv[0]);
+    std::fprintf(stderr, "usage: %s <fusion.yaml> <kernels.yaml> <File name | index | all> [--preset P] [--split N] [--iters N] [--small]\n", argv[0]);
     return 2;
   }
   std::string preset = "hfuse";
@@ -275,52 +321,34 @@ int main(int argc, char **argv) {
   try {
     hf_config *cfg = nullptr;
     hf_check(hf_config_load_files(argv[1], argv[2], &cfg));
-    int index = -1;
-    const char *file = "", *k1 = "", *k2 = "";
-    for (int i = 0; i < hf_config_num_fusions(cfg); i++) {
+    const std::string which = argv[3];
+    const int n = hf_config_num_fusions(cfg);
+    std::vector<int> todo;
+    for (int i = 0; i < n; i++) {
+      const char *file = "", *k1 = "", *k2 = "";
       hf_check(hf_config_fusion(cfg, i, &file, &k1, &k2));
-      if (std::string(argv[3]) == file || std::to_string(i) == argv[3]) { index = i; break; }
+      if (which == "all" ? hf_config_fusion_size(cfg, i) == 2 : (which == file || std::to_string(i) == which)) {
+        todo.push_back(i);
+        if (which != "all") break;
+      }
     }
-    if (index < 0) throw std::runtime_error(std::string("no fusion '") + argv[3] + "' in " + argv[1]);
-    hf_plan *plan = nullptr;
-    hf_check(hf_plan_create(cfg, index, preset.c_str(), split, 0, &plan));
-    hf_partition part;
-    hf_check(hf_plan_partition(plan, &part));
-    std::printf("%s: %s + %s as %s (%u threads: [%u,%u) + [%u,%u))\n", file, k1, k2, part.name, part.launch_threads,
-                part.lo[0], part.hi[0], part.lo[1], part.hi[1]);
-
-    const bool hist_pair = std::string(k1) == "kernelHistogram1D";
-    auto w1 = make_workload(k1, false, small, 0x48467573ull);
-    auto w2 = make_workload(k2, hist_pair, small, 0x48467574ull);
-    // ethash scans grid * (its block) nonces: natively 128-thread blocks, fused its share of the block
-    const int native_grid = w1->grid ? w1->grid : w2->grid;
-    int fused_grid = 0;
-    if (w1->grid) fused_grid = (int)(w1->hashes / (part.hi[0] - part.lo[0]));
-    if (w2->grid) fused_grid = (int)(w2->hashes / (part.hi[1] - part.lo[1]));
-
-    // one compared launch of each form on identical inputs
-    w1->reset();
-    w2->reset();
-    hip_check(hipDeviceSynchronize(), "reset");
-    hf_check(hf_launch_native(k1, w1->args_native.data(), w1->grid, 0, nullptr));
-    hf_check(hf_launch_native(k2, w2->args_native.data(), w2->grid, 0, nullptr));
-    hf_check(hf_launch_fused(plan, w1->args_fused.data(), w2->args_fused.data(), fused_grid, nullptr));
-    hip_check(hipDeviceSynchronize(), "compared launches");
-    const bool ok1 = same_outputs(*w1), ok2 = same_outputs(*w2);
-    std::printf("fused == native: %s %s, %s %s\n", k1, ok1 ? "yes" : "NO", k2, ok2 ? "yes" : "NO");  // batch-norm: to 1e-5 relative
-
-    // timed repetitions: A, B, A then B, fused
-    const void *a1[1] = {w1->args_native.data()}, *a2[1] = {w2->args_native.data()};
-    const char *label[4] = {k1, k2, "back to back", part.name};
-    float ms[4];
-    for (int mode = 0; mode < 4; mode++) {
-      hf_check(hf_time_pair(plan, mode, a1, a2, 1, 2, iters, mode == 3 ? fused_grid : native_grid, nullptr, &ms[mode]));
-      std::printf("%-60s %10.3f us per launch\n", label[mode], 1e3 * ms[mode] / iters);
+    if (todo.empty()) throw std::runtime_error("no fusion '" + which + "' in " + argv[1]);
+    bool all_ok = true;
+    std::vector<std::pair<std::string, double>> summary;
+    for (int index : todo) {
+      bool ok = false;
+      const double speedup = run_pair(cfg, index, preset, split, iters, small, ok);
+      all_ok = all_ok && ok;
+      const char *file = "", *k1 = "", *k2 = "";
+      hf_check(hf_config_fusion(cfg, index, &file, &k1, &k2));
+      summary.emplace_back(std::string(file) + (ok ? "" : "  (OUTPUTS DIFFER)"), speedup);
     }
-    std::printf("speedup of the fused kernel over back to back: %+.1f %%\n", (ms[2] / ms[3] - 1.0) * 100.0);
-    hf_plan_free(plan);
+    if (todo.size() > 1) {
+      std::printf("\n%-40s %s\n", "pair", "fused over back to back");
+      for (const auto &row : summary) std::printf("%-40s %+6.1f %%\n", row.first.c_str(), row.second);
+    }
     hf_config_free(cfg);
-    return ok1 && ok2 ? 0 : 1;
+    return all_ok ? 0 : 1;
   } catch (const std::exception &e) {
     std::fprintf(stderr, "hfuse-launch: %s\n", e.what());
     return 1;

@@ -37,6 +37,14 @@ def test_benchmark_shapes(cuda, pair):
     assert r.stdout.count(" yes") == 2
 
 
+def test_all_pairs_in_one_run(cuda):
+    r = run("all", "--small", "--iters", "2")
+    assert r.returncode == 0, (r.stdout[-2000:], r.stderr)
+    cfg = hfuse_amd.default_config()
+    assert r.stdout.count("fused == native:") == cfg.num_fusions
+    assert " NO" not in r.stdout and "fused over back to back" in r.stdout
+
+
 def test_errors(cuda):
     assert run("NoSuchPair").returncode == 1
     assert run("0", "--preset", "hfuse_bar_sync").returncode == 1
