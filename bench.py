@@ -226,7 +226,6 @@ def cpu_baseline_tensor(name, budget_s=12.0):
     """Oracle (C port, OpenMP) and PyTorch CPU ops on the full shape of the pair, repeated within a budget."""
     import torch
     from oracle import oracle as O
-    import numpy as np
     g = torch.Generator().manual_seed(1)
     if name == "bn_upsample":
         x = (torch.randn((32, 256, 28, 28), generator=g) * 2 + 0.5).contiguous()

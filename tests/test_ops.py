@@ -1,5 +1,4 @@
 """The torch-tensor operator layer: same results as the PyTorch CPU operators the oracle is pinned to."""
-import numpy as np
 import pytest
 import torch
 import torch.nn.functional as F
