@@ -18,6 +18,19 @@ enum { HINT_GENERIC = 0, HINT_IM2COL_3X3_S1P1 = 1, HINT_POOL_K3S2P1 = 1, HINT_PO
        HINT_IDX32 = 0x100 };
 
 __device__ __forceinline__ f32x4 ld4(const float *p) { return *reinterpret_cast<const f32x4 *>(p); }
+// The same load with the non-temporal hint, for streams whose every byte is read once (the histogram's
+// input, 2x2 pooling windows): they then leave the caches to whoever re-reads.  Kernels that do re-read
+// through the cache (im2col's taps, overlapping 3x3 windows) lose 10-30 % with it.
+#ifndef HF_NT_LOADS
+#define HF_NT_LOADS 1
+#endif
+__device__ __forceinline__ f32x4 ld4_stream(const float *p) {
+#if HF_NT_LOADS
+  return __builtin_nontemporal_load(reinterpret_cast<const f32x4 *>(p));
+#else
+  return *reinterpret_cast<const f32x4 *>(p);
+#endif
+}
 
 // One DPP move of a float.  0x138 = wave_shr:1 (lane i receives lane i-1's value),
 // 0x130 = wave_shl:1 (lane i receives lane i+1's); the lane without a source keeps 0.
@@ -229,7 +242,7 @@ struct MaxPoolBody {
         const int h = hstart + i;
         const bool in = h >= 0 && h < (int)H;
         const float *row = plane + (unsigned)(in ? h : h0) * W + wbase;
-        v[i] = ld4(row);
+        v[i] = (K == 2 && P == 0) ? ld4_stream(row) : ld4(row);
         left[i] = (P == 1 && wbase > 0) ? row[-1] : 0.0f;
       }
 #pragma unroll
@@ -735,11 +748,11 @@ struct HistcBody {
       for (; i + (HF_HIST_U - 1) * stride < n4; i += HF_HIST_U * stride) {
         f32x4 v[HF_HIST_U];
 #pragma unroll
-        for (int u = 0; u < HF_HIST_U; u++) v[u] = ld4(b + (i + u * stride) * 4);
+        for (int u = 0; u < HF_HIST_U; u++) v[u] = ld4_stream(b + (i + u * stride) * 4);
 #pragma unroll
         for (int u = 0; u < HF_HIST_U; u++) count4(v[u]);
       }
-      for (; i < n4; i += stride) count4(ld4(b + i * 4));
+      for (; i < n4; i += stride) count4(ld4_stream(b + i * 4));
       if (sb.bid == 0)
         for (int64_t k = (n4 << 2) + sb.tid; k < rest; k += sb.nthreads)
           count<POW2, GLOBAL>(bins, b[k], lo, hi, fn, range, inv_range, inv_lo, inv_hi, nbins);
