@@ -369,7 +369,7 @@ struct EthashBody {
           }
           u32x4 item[kParallel];
 #pragma unroll
-          for (int p = 0; p < kParallel; p++) item[p] = a.dag[(size_t)offset[p] * 8 + lane_in_group];
+          for (int p = 0; p < kParallel; p++) item[p] = __builtin_nontemporal_load(a.dag + (size_t)offset[p] * 8 + lane_in_group);
 #pragma unroll
           for (int p = 0; p < kParallel; p++) mix[p] = fnv4(mix[p], item[p]);
         }

@@ -239,6 +239,9 @@ def main(argv=None) -> int:
     ap.add_argument("--only", default="", help="comma list of File names or k1+k2 to tune (default: every tensor pair)")
     ap.add_argument("--searches", action="store_true", help="also tune the nonce-search pairs (allocates a 4 GiB DAG)")
     ap.add_argument("--search-log2", type=int, default=24, help="log2 of the nonce range of a search launch while tuning")
+    ap.add_argument("--search-log2-second", type=int, default=None,
+                    help="log2 of the second kernel's nonce range (default: the same as --search-log2); the benchmark's "
+                         "Ethash + Blake2b pair runs 2^28 against 2^30 nonces, i.e. a difference of 2")
     ap.add_argument("--step", type=int, default=64, help="granule of the block-shape sweep in threads")
     ap.add_argument("--min-gain", type=float, default=1.0,
                     help="keep an entry's current keys unless the winner beats the table split by this many percent")
@@ -281,7 +284,8 @@ def main(argv=None) -> int:
                      barrier_modes=(None, L.HF_BARRIER_BLOCKIDX) if args.blockidx else (None,), verbose=args.verbose)
             del pair
         else:
-            sp = W.SearchPair(k1, k2, args.search_log2, args.search_log2)
+            sp = W.SearchPair(k1, k2, args.search_log2,
+                              args.search_log2 if args.search_log2_second is None else args.search_log2_second)
             _, _, a1, a2 = sp.fresh()
             # ethash scans grid * its-threads nonces: every block shape gets the grid for the same range
             eth = 0 if k1 == "ethash_search" else 1 if k2 == "ethash_search" else None
