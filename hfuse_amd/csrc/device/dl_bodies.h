@@ -19,7 +19,7 @@ enum { HINT_GENERIC = 0, HINT_IM2COL_3X3_S1P1 = 1, HINT_POOL_K3S2P1 = 1, HINT_PO
 
 __device__ __forceinline__ f32x4 ld4(const float *p) { return *reinterpret_cast<const f32x4 *>(p); }
 // The same load with the non-temporal hint, for streams whose every byte is read once (the histogram's
-// input, 2x2 pooling windows): they then leave the caches to whoever re-reads.  Kernels that do re-read
+// input, batch-norm planes, 2x2 pooling windows): they then leave the caches to whoever re-reads.  Kernels that do re-read
 // through the cache (im2col's taps, overlapping 3x3 windows) lose 10-30 % with it.
 #ifndef HF_NT_LOADS
 #define HF_NT_LOADS 1
@@ -613,7 +613,7 @@ struct BnStatsBody {
         };
         auto chunk = [&](unsigned ch) {
           const unsigned b = ch / lq, q = ch - b * lq;
-          return ld4(base + (size_t)b * a.input.strides[0] + (size_t)q * 4);
+          return ld4_stream(base + (size_t)b * a.input.strides[0] + (size_t)q * 4);
         };
 #ifndef HF_BN_U
 #define HF_BN_U 4
