@@ -34,7 +34,7 @@ class Dim3(C.Structure):
 
 class KernelInfo(C.Structure):
     _fields_ = [("kernel_name", C.c_char * 96), ("has_barriers", C.c_int), ("block_dim", Dim3),
-                ("reg", C.c_uint32), ("exec_time", C.c_double)]
+                ("reg", C.c_uint32), ("exec_time", C.c_double), ("native_threads", C.c_uint32)]
 
 
 class Partition(C.Structure):

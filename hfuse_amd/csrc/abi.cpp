@@ -609,6 +609,7 @@ HF_API int hf_config_kernel(const hf_config *cfg, const char *name, hf_kernel_in
   out->block_dim = {r->block_dim.x, r->block_dim.y, r->block_dim.z};
   out->reg = r->reg;
   out->exec_time = r->exec_time;
+  out->native_threads = r->native_block();
   return HF_OK;
 } catch (...) {
   return trap_exception();
@@ -865,7 +866,8 @@ HF_API int hf_launch_native(const char *kernel_name, const void *args, int grid_
   Prepared p;
   int rc = prepare(id, args, p);
   if (rc != HF_OK) return rc;
-  unsigned block = block_threads > 0 ? (unsigned)block_threads : (is_crypto(id) ? 128u : (id == K_MAXPOOL ? 256u : 512u));
+  unsigned block = block_threads > 0 ? (unsigned)block_threads
+                                     : (is_crypto(id) ? 128u : (id == K_MAXPOOL ? 256u : (id == K_HISTC ? 768u : 512u)));
   return do_launch_native(id, p, grid_blocks, block, static_cast<hipStream_t>(stream));
 } catch (...) {
   return trap_exception();
@@ -994,7 +996,7 @@ HF_API int hf_time_pair(const hf_plan *plan, int mode, const void *const *args1,
     rc = prepare(plan->ids[1], args2[i], p2[i]);
     if (rc != HF_OK) return rc;
   }
-  const unsigned b1 = plan->rows[0].block_dim.size(), b2 = plan->rows[1].block_dim.size();
+  const unsigned b1 = plan->rows[0].native_block(), b2 = plan->rows[1].native_block();
   auto once = [&](int i) -> int {
     const int s = i % nsets;
     int rc = HF_OK;

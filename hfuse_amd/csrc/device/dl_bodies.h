@@ -7,6 +7,8 @@
 #pragma once
 #include <hip/hip_runtime.h>
 
+#include <type_traits>
+
 #include "../../../include/hfuse_gfx950.h"
 #include "subblock.h"
 
@@ -741,17 +743,21 @@ struct HistcBody {
       const int64_t n4 = rest >> 2;
       const int64_t stride = (int64_t)sb.gstride();
       int64_t i = (int64_t)sb.gtid();
-      // several 16-byte loads in flight per lane before the dependent LDS atomics
-#ifndef HF_HIST_U
-#define HF_HIST_U 8
-#endif
-      for (; i + (HF_HIST_U - 1) * stride < n4; i += HF_HIST_U * stride) {
-        f32x4 v[HF_HIST_U];
+      // Several 16-byte loads in flight per lane before the dependent LDS atomics: eight with up to
+      // eight wavefronts, four with more (about 48-64 KB in flight per CU either way; beyond that the
+      // memory system gets slower, and more wavefronts with shorter batches overlap their arithmetic better).
+      auto batches = [&](auto unroll) {
+        constexpr int U = decltype(unroll)::value;
+        for (; i + (U - 1) * stride < n4; i += U * stride) {
+          f32x4 v[U];
 #pragma unroll
-        for (int u = 0; u < HF_HIST_U; u++) v[u] = ld4_stream(b + (i + u * stride) * 4);
+          for (int u = 0; u < U; u++) v[u] = ld4_stream(b + (i + u * stride) * 4);
 #pragma unroll
-        for (int u = 0; u < HF_HIST_U; u++) count4(v[u]);
-      }
+          for (int u = 0; u < U; u++) count4(v[u]);
+        }
+      };
+      if (sb.nthreads > 512) batches(std::integral_constant<int, 4>());
+      else batches(std::integral_constant<int, 8>());
       for (; i < n4; i += stride) count4(ld4_stream(b + i * 4));
       if (sb.bid == 0)
         for (int64_t k = (n4 << 2) + sb.tid; k < rest; k += sb.nthreads)

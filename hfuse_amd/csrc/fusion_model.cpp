@@ -81,9 +81,19 @@ bool parse_row(const YamlNode &n, bool reg_required, KernelRow &row, std::string
       return false;
     }
   }
+  // Not in the reference's schema: the block the unfused kernel is launched with on this GPU, where that
+  // is not BlockDim (which stays the basis of the split enumeration and must keep pair totals within 1024).
+  if (const YamlNode *nt = n.get("NativeThreads")) {
+    if (!to_uint(nt, row.native_threads) || row.native_threads == 0 || row.native_threads % kWave != 0 ||
+        row.native_threads > kMaxBlock) {
+      err = at(*nt) + "'NativeThreads' must be a multiple of 64 between 64 and 1024";
+      return false;
+    }
+  }
   for (auto &kv : n.map) {
     const std::string &k = kv.first;
-    if (k != "KernelName" && k != "HasBarriers" && k != "BlockDim" && k != "Reg" && k != "ExecTime") {
+    if (k != "KernelName" && k != "HasBarriers" && k != "BlockDim" && k != "Reg" && k != "ExecTime" &&
+        k != "NativeThreads") {
       err = at(kv.second) + "unknown key '" + k + "'";
       return false;
     }

@@ -23,6 +23,8 @@ struct KernelRow {
   Dim3 block_dim;
   uint32_t reg = 0;
   double exec_time = -1.0;
+  uint32_t native_threads = 0;  // optional `NativeThreads:` key: block of the unfused launch when it is not BlockDim's product
+  uint32_t native_block() const { return native_threads ? native_threads : block_dim.x * block_dim.y * block_dim.z; }
 };
 
 struct FusionRow {

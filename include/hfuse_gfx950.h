@@ -68,6 +68,7 @@ typedef struct {
   hf_dim3 block_dim;
   uint32_t reg;
   double exec_time; /* -1 when the YAML has no ExecTime */
+  uint32_t native_threads; /* block of the unfused launch: BlockDim's product unless the row has NativeThreads */
 } hf_kernel_info;
 
 /*
@@ -84,6 +85,10 @@ typedef struct {
  * for hf_plan_set_lending and `Barrier: none|matched|subset|blockidx` the one
  * for hf_plan_set_barrier_mode (an illegal mode fails hf_plan_create);
  * `LaunchBound: true|false` the one for hf_plan_set_launch_bound.
+ * A kernel row may carry one extra key, `NativeThreads: <threads>` (a multiple of 64, at most 1024): the
+ * block the unfused kernel is launched with by hf_time_pair when that differs from BlockDim, which stays
+ * the basis of the split enumeration (the histogram runs fastest alone at 768 threads, and BlockDim 768
+ * would push its pairs' totals d1 + d2 beyond 1024).
  */
 HF_API int hf_config_load_text(const char *fusion_yaml, const char *kernels_yaml, hf_config **out);
 HF_API int hf_config_load_files(const char *fusion_path, const char *kernels_path, hf_config **out);

@@ -510,3 +510,20 @@ def test_partition_matches_oracle_on_random_kernel_tables():
             assert got.launch_threads == want.launch_threads and got.launch_blocks == want.launch_blocks
             checked += 1
     assert checked > 800 and refused > 10
+
+
+def test_native_threads_key():
+    """`NativeThreads` (not in the reference's schema) names the block of the unfused launch; BlockDim stays
+    the basis of the split enumeration."""
+    row = "k:\n  KernelName: kernelHistogram1D\n  HasBarriers: true\n  BlockDim:\n    X: 512\n    Y: 1\n    Z: 1\n  Reg: 19\n"
+    fusion = "- File: f\n  Kernels:\n    - k\n    - k\n"
+    cfg = Config(fusion, row + "  NativeThreads: 768\n")
+    info = cfg.kernel("k")
+    assert info.native_threads == 768 and info.block_dim.x == 512
+    assert Config(fusion, row).kernel("k").native_threads == 512
+    assert cfg.num_splits(0) == 7                       # 128 * (n + 1) < 512 + 512, whatever the native block
+    for bad in ("0", "100", "2048", "many"):
+        with pytest.raises(hfuse_amd.HfuseError) as e:
+            Config(fusion, row + f"  NativeThreads: {bad}\n")
+        assert e.value.code == L.HF_EPARSE and "NativeThreads" in e.value.message
+    assert hfuse_amd.default_config().kernel("kernelHistogram1D").native_threads == 768
