@@ -36,6 +36,11 @@ __device__ __forceinline__ f32x4 ld4_stream(const float *p) {
 
 // One DPP move of a float.  0x138 = wave_shr:1 (lane i receives lane i-1's value),
 // 0x130 = wave_shl:1 (lane i receives lane i+1's); the lane without a source keeps 0.
+// The first active lane's value of a 64-bit quantity, as a wave-uniform value.
+__device__ __forceinline__ size_t uniform_u64(size_t x) {
+  return ((size_t)__builtin_amdgcn_readfirstlane((unsigned)(x >> 32)) << 32) | (unsigned)__builtin_amdgcn_readfirstlane((unsigned)x);
+}
+
 template <int CTRL>
 __device__ __forceinline__ float dpp_f32(float v) {
   return __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), CTRL, 0xF, 0xF, false));
@@ -245,7 +250,23 @@ struct MaxPoolBody {
         const bool in = h >= 0 && h < (int)H;
         const float *row = plane + (unsigned)(in ? h : h0) * W + wbase;
         v[i] = (K == 2 && P == 0) ? ld4_stream(row) : ld4(row);
-        left[i] = (P == 1 && wbase > 0) ? row[-1] : 0.0f;
+        left[i] = 0.0f;
+        if constexpr (P == 1) {
+          // Lane 0 has nobody to its left in this wavefront: its column wbase - 1 is loaded from an
+          // address every lane agrees on (one cache line, no divergence).  In column 0 it is padding.
+          const size_t off = (size_t)(row - a.bottom_data);
+          left[i] = a.bottom_data[uniform_u64(wbase > 0 ? off - 1 : off)];
+        }
+      }
+      if constexpr (P == 1) {
+        // Column wbase - 1 is the last column of the lane to the left (neighbouring lanes hold
+        // neighbouring work items; with wbase > 0 they sit in the same output row and loaded the
+        // same input rows), so it comes by a wavefront shift instead of a second load per row.
+#pragma unroll
+        for (int i = 0; i < K; i++) {
+          const float from_left = dpp_f32<0x138>(v[i].w);
+          if (sb.lane() != 0) left[i] = from_left;
+        }
       }
 #pragma unroll
       for (int i = 0; i < K; i++) {
