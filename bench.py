@@ -28,7 +28,7 @@ HBM_PEAK_GBPS = 8000.0            # MI355X HBM3E
 VALU_PEAK_GOPS = 256 * 128 * 2.4  # 256 CUs x 128 lanes x 2.4 GHz int32 op/s in Gop/s (= 157.3 TFLOP/s fp32 / 2)
 # HBM bytes per launch of the headline fused kernel from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE, each
 # scaled by what the same counter reads for the plain copy kernel (profiles/tensor_pairs_hbm_traffic.md)
-HEADLINE_TRAFFIC_BYTES = {"bn_upsample": 157.05e6, "im2col_maxpool": 443.23e6, "histc_maxpool": 329.49e6}
+HEADLINE_TRAFFIC_BYTES = {"bn_upsample": 156.98e6, "im2col_maxpool": 443.28e6, "histc_maxpool": 329.49e6}
 
 # textbook primitive-op counts per hash (add / logic / rotate / shift = 1 each)
 OPS_SHA256D = 4336
