@@ -700,7 +700,7 @@ struct HistcBody {
       const float t = (v - lo) * scale_n;
       int bin;
       if constexpr (POW2) {
-        bin = (int)(t * inv_range);
+        bin = (int)t;  // scale_n already holds nbins / range: scaling by a power of two commutes with rounding
       } else {
         // (int)(t / range) without the division where that is safe.  t times two reciprocals that
         // bracket 1 / range by a relative 2^-21 brackets the correctly rounded quotient; when both
@@ -714,7 +714,7 @@ struct HistcBody {
           if (unsure) bin = (int)(t / range);
         }
       }
-      if (bin == nbins) bin -= 1;
+      bin = min(bin, nbins - 1);  // v == max lands in bin nbins: the original's `if (bin == nbins) bin -= 1`
       if constexpr (GLOBAL) unsafeAtomicAdd(reinterpret_cast<float *>(bins) + bin, 1.0f);
       else __hip_atomic_fetch_add(bins + bin, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
     }
@@ -743,8 +743,10 @@ struct HistcBody {
     if constexpr (!GLOBAL)
       for (int i = (int)sb.tid; i < nbins; i += (int)sb.nthreads) bins[i] = 0;
     sb.sync();
-    const float lo = a.minvalue, hi = a.maxvalue, range = hi - lo, fn = (float)nbins;
+    const float lo = a.minvalue, hi = a.maxvalue, range = hi - lo;
     const float inv_range = 1.0f / range;
+    // (v - lo) * nbins / range: with a power-of-two range the division is an exact scaling, folded into the factor
+    const float fn = POW2 ? (float)nbins * inv_range : (float)nbins;
     const float inv_lo = inv_range * (1.0f - 0x1p-21f), inv_hi = inv_range * (1.0f + 0x1p-21f);
     const float *b = a.b.data;
     const int64_t total = a.total_elements;

@@ -329,7 +329,10 @@ def test_histc_unaligned_input(cuda, offset, n):
 
 
 @pytest.mark.parametrize("nbins,lo,hi", [(1000, 0.0, 3.0), (7, -0.7, 0.0), (15360, 0.0, 10.0), (1024, 0.1, 0.9),
-                                         (100, -5.0, 123.0), (3, 1e-3, 1e3), (1024, 0.0, 1.0)])
+                                         (100, -5.0, 123.0), (3, 1e-3, 1e3), (1024, 0.0, 1.0),
+                                         # power-of-two widths (the division is folded into the scale factor)
+                                         (1000, -3.0, 5.0), (777, 0.25, 0.75), (15360, -1.0, 1.0), (5, 0.0, 2.0 ** -20),
+                                         (1023, -2.0 ** 20, 2.0 ** 20)])
 def test_histc_bin_edges_with_any_range(cuda, nbins, lo, hi):
     """Ranges whose width is not a power of two go through the real fp32 division of the bin
     formula.  The inputs sit on and one ulp either side of every bin edge (where the rounding
