@@ -372,7 +372,8 @@ HF_API int hf_blake2b_set_block(const uint8_t header[80], void *stream);
 /*
  * Native launch of one original kernel by its YAML name; `args` points at the
  * matching hf_*_args.  grid_blocks <= 0 lets the library size the grid from the
- * work; block threads come from block_threads (<= 0: the kernel's default).
+ * work; block threads come from block_threads (<= 0: the kernel's default --
+ * 128 for the searches, 256 for max-pooling, 768 for the histogram, 512 otherwise).
  */
 HF_API int hf_launch_native(const char *kernel_name, const void *args, int grid_blocks,
                             int block_threads, void *stream);
