@@ -147,7 +147,15 @@ PROTOTYPES = {
     "hf_sha256d_set_block": (C.c_int, [C.c_char_p, C.c_uint64, C.c_void_p]),
     "hf_sia_blake2b_set_block": (C.c_int, [C.c_char_p, C.c_void_p]),
     "hf_blake2b_set_block": (C.c_int, [C.c_char_p, C.c_void_p]),
+    "hf_constants_create": (C.c_int, [C.POINTER(C.c_void_p)]),
+    "hf_constants_free": (None, [C.c_void_p]),
+    "hf_constants_set_ethash": (C.c_int, [C.c_void_p, C.c_void_p, C.c_uint32, C.c_char_p, C.c_uint64]),
+    "hf_constants_set_sha256d": (C.c_int, [C.c_void_p, C.c_char_p, C.c_uint64]),
+    "hf_constants_set_sia_blake2b": (C.c_int, [C.c_void_p, C.c_char_p]),
+    "hf_constants_set_blake2b": (C.c_int, [C.c_void_p, C.c_char_p]),
+    "hf_plan_bind_constants": (C.c_int, [C.c_void_p, C.c_void_p]),
     "hf_launch_native": (C.c_int, [C.c_char_p, C.c_void_p, C.c_int, C.c_int, C.c_void_p]),
+    "hf_launch_native_with": (C.c_int, [C.c_char_p, C.c_void_p, C.c_void_p, C.c_int, C.c_int, C.c_void_p]),
     "hf_launch_fused": (C.c_int, [C.c_void_p, C.c_void_p, C.c_void_p, C.c_int, C.c_void_p]),
     "hf_time_pair": (C.c_int, [C.c_void_p, C.c_int, C.POINTER(C.c_void_p), C.POINTER(C.c_void_p), C.c_int,
                                C.c_int, C.c_int, C.c_int, C.c_void_p, C.POINTER(C.c_float)]),

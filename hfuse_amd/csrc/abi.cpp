@@ -90,8 +90,10 @@ bool body_has_barriers(KernelId id) { return id == K_BNSTATS || id == K_HISTC; }
 bool body_is_flat(KernelId id) { return id != K_BNSTATS && id != K_HISTC && id != K_ETHASH; }
 
 // ------------------------------------------------ constants of the searches
+// What the original kernels read from __constant__ symbols.  One process-wide set mirrors those
+// symbols (hf_*_set_*); an hf_constants object is a caller-owned set that a plan can be bound to
+// or a native launch can name, so that host threads working on different headers never share state.
 struct SearchConstants {
-  std::mutex mu;
   // ethash
   const void *dag = nullptr;
   uint32_t dag_items = 0;
@@ -99,16 +101,23 @@ struct SearchConstants {
   uint64_t eth_target = 0;
   bool eth_set = false;
   // sha256d
-  uint32_t sha_mid[8];
-  uint32_t sha_tail[3];
+  uint32_t sha_mid[8] = {0};
+  uint32_t sha_tail[3] = {0};
   uint64_t sha_target = 0;
   bool sha_set = false;
   // blake2b headers
-  uint64_t sia_m[10];
+  uint64_t sia_m[10] = {0};
   bool sia_set = false;
-  uint64_t b2_m[10];
+  uint64_t b2_m[10] = {0};
   bool b2_set = false;
-} g_const;
+};
+std::mutex g_const_mu;      // guards g_const only
+SearchConstants g_const;    // the process-wide set
+
+SearchConstants snapshot_process_constants() {
+  std::lock_guard<std::mutex> lock(g_const_mu);
+  return g_const;
+}
 
 uint32_t load_be32(const uint8_t *p) {
   return ((uint32_t)p[0] << 24) | ((uint32_t)p[1] << 16) | ((uint32_t)p[2] << 8) | p[3];
@@ -169,6 +178,7 @@ struct Prepared {
   unsigned hint = 0;
   unsigned lds = 0;
   bool exact_grid = false;  // the grid decides the amount of work (ethash)
+  bool idx32 = false;       // the chosen path walks its work items with a 32-bit counter
   unsigned long long items = 0;  // work items of one pass at the chosen hint
 };
 
@@ -225,6 +235,7 @@ int prepare_im2col(const hf_im2col_args &a, Prepared &p) {
                      a.height_col * a.stride_h < lim && a.width_col * a.stride_w < lim;
   p.hint = fast ? HINT_IM2COL_3X3_S1P1 : idx32 ? HINT_IDX32 : HINT_GENERIC;
   p.items = fast ? (unsigned long long)a.n / 4 : (unsigned long long)a.n;
+  p.idx32 = p.hint != HINT_GENERIC;
   return HF_OK;
 }
 
@@ -260,6 +271,7 @@ int prepare_maxpool(const hf_maxpool_args &a, Prepared &p) {
     p.hint = HINT_POOL_K2S2P0;
   p.items = (p.hint == HINT_POOL_K3S2P1 || p.hint == HINT_POOL_K2S2P0) ? (unsigned long long)a.nthreads / 2
                                                                          : (unsigned long long)a.nthreads;
+  p.idx32 = p.hint != HINT_GENERIC;
   return HF_OK;
 }
 
@@ -314,6 +326,7 @@ int prepare_upsample(const hf_upsample_nearest_args &a, Prepared &p) {
                     out_elems < (int64_t)1 << 32;
   p.hint = fast ? HINT_UP_2X : (in_elems < (int64_t)1 << 31 && out_elems < (int64_t)1 << 31) ? HINT_IDX32 : HINT_GENERIC;
   p.items = fast ? (unsigned long long)in_elems / 2 : (unsigned long long)out_elems;
+  p.idx32 = p.hint != HINT_GENERIC;
   return HF_OK;
 }
 
@@ -331,7 +344,26 @@ int prepare_bilinear(const hf_upsample_bilinear_args &a, Prepared &p) {
     return fail(HF_EUNSUPPORTED, std::string(who) + "tensors of 2^32 elements or more are not built");
   if (!product(hw, {a.odata.sizes[2], a.odata.sizes[3]}) || (int64_t)a.n != hw)
     return fail(HF_EINVAL, std::string(who) + "n is not height2 * width2");
-  if (!(a.rheight >= 0.0f) || !(a.rwidth >= 0.0f)) return fail(HF_EINVAL, std::string(who) + "negative scale");
+  if (!(a.rheight >= 0.0f) || !(a.rwidth >= 0.0f) || !std::isfinite(a.rheight) || !std::isfinite(a.rwidth))
+    return fail(HF_EINVAL, std::string(who) + "scales must be finite and not negative");
+  // The kernel reads input row (int)src and column (int)src of every output pixel without a clamp,
+  // as the original does: the source index of the last output row / column, evaluated in the
+  // kernel's own fp32 steps (it grows with the destination index), must lie inside the input.
+  auto last_source = [&](float scale, int64_t out_size) {
+    const volatile float dst = (float)(out_size - 1);
+    if (a.align_corners) {
+      const volatile float s = scale * dst;
+      return (double)s;
+    }
+    const volatile float t0 = dst + 0.5f;
+    const volatile float t1 = scale * t0;
+    const volatile float t2 = t1 - 0.5f;
+    return (double)(t2 < 0.0f ? 0.0f : t2);
+  };
+  const bool same_size = a.idata.sizes[2] == a.odata.sizes[2] && a.idata.sizes[3] == a.odata.sizes[3];  // a plain copy
+  if (!same_size && (last_source(a.rheight, a.odata.sizes[2]) >= (double)a.idata.sizes[2] ||
+                     last_source(a.rwidth, a.odata.sizes[3]) >= (double)a.idata.sizes[3]))
+    return fail(HF_EINVAL, std::string(who) + "scale maps the last output row or column beyond the input");
   for (const hf_accessor4 *t : {&a.idata, &a.odata}) {
     int64_t reach = 0;
     for (int i = 0; i < 4; i++) {
@@ -355,6 +387,7 @@ int prepare_bilinear(const hf_upsample_bilinear_args &a, Prepared &p) {
                      a.odata.sizes[2] < (1 << 22) && a.odata.sizes[3] < (1 << 22);
   p.hint = twice ? HINT_BILINEAR_2X : fast ? HINT_BILINEAR_VEC4 : HINT_GENERIC;
   p.items = twice ? (unsigned long long)total / 8 : fast ? (unsigned long long)total / 4 : (unsigned long long)total;
+  p.idx32 = true;  // every bilinear path counts in 32 bits (tensors below 2^32 elements)
   return HF_OK;
 }
 
@@ -389,61 +422,64 @@ int prepare_histc(const hf_histc_args &a, Prepared &p) {
   return HF_OK;
 }
 
-int prepare_ethash(const hf_ethash_args &a, Prepared &p) {
+int prepare_ethash(const hf_ethash_args &a, const SearchConstants &c, Prepared &p) {
   if (!a.g_output) return fail(HF_EINVAL, "ethash_search: null result pointer");
-  std::lock_guard<std::mutex> lock(g_const.mu);
-  if (!g_const.eth_set) return fail(HF_EINVAL, "ethash_search: hf_ethash_set_constants has not been called");
+  if (!c.eth_set) return fail(HF_EINVAL, "ethash_search: hf_ethash_set_constants has not been called");
   EthashDevArgs d;
   d.out = a.g_output;
   d.start_nonce = a.start_nonce;
-  d.dag = static_cast<const u32x4 *>(g_const.dag);
-  d.n_items = g_const.dag_items;
+  d.dag = static_cast<const u32x4 *>(c.dag);
+  d.n_items = c.dag_items;
   d.pow2_mask = (d.n_items & (d.n_items - 1)) == 0 ? d.n_items - 1 : 0;
-  d.target = g_const.eth_target;
-  std::memcpy(d.header, g_const.eth_header, sizeof d.header);
+  d.target = c.eth_target;
+  std::memcpy(d.header, c.eth_header, sizeof d.header);
   std::memcpy(p.blob, &d, sizeof d);
   p.exact_grid = true;
   return HF_OK;
 }
 
-int prepare_sha256d(const hf_sha256d_args &a, Prepared &p) {
+int prepare_sha256d(const hf_sha256d_args &a, const SearchConstants &c, Prepared &p) {
   if (!a.res_nonces) return fail(HF_EINVAL, "sha256d_gpu_hash_shared: null result pointer");
-  std::lock_guard<std::mutex> lock(g_const.mu);
-  if (!g_const.sha_set) return fail(HF_EINVAL, "sha256d_gpu_hash_shared: hf_sha256d_set_block has not been called");
+  if (!c.sha_set) return fail(HF_EINVAL, "sha256d_gpu_hash_shared: hf_sha256d_set_block has not been called");
   Sha256dDevArgs d;
   d.threads = a.threads;
   d.start_nonce = a.start_nonce;
   d.out = reinterpret_cast<hf_search_results *>(a.res_nonces);
-  std::memcpy(d.midstate, g_const.sha_mid, sizeof d.midstate);
-  std::memcpy(d.tail, g_const.sha_tail, sizeof d.tail);
+  std::memcpy(d.midstate, c.sha_mid, sizeof d.midstate);
+  std::memcpy(d.tail, c.sha_tail, sizeof d.tail);
   d.pad = 0;
-  d.target64 = g_const.sha_target;
+  d.target64 = c.sha_target;
   std::memcpy(p.blob, &d, sizeof d);
   p.items = a.threads;
   return HF_OK;
 }
 
-int prepare_blake2b(const hf_blake2b_args &a, bool sia, Prepared &p) {
+int prepare_blake2b(const hf_blake2b_args &a, bool sia, const SearchConstants &c, Prepared &p) {
   const char *who = sia ? "sia_blake2b_gpu_hash" : "blake2b_gpu_hash";
   if (!a.res_nonce) return fail(HF_EINVAL, std::string(who) + ": null result pointer");
-  std::lock_guard<std::mutex> lock(g_const.mu);
-  if (!(sia ? g_const.sia_set : g_const.b2_set))
+  if (!(sia ? c.sia_set : c.b2_set))
     return fail(HF_EINVAL, std::string(who) + ": the header block has not been set");
   Blake2bDevArgs d;
   d.threads = a.threads;
   d.start_nonce = a.start_nonce;
   d.out = reinterpret_cast<hf_search_results *>(a.res_nonce);
   d.target64 = ((uint64_t)a.target2[1] << 32) | a.target2[0];
-  std::memcpy(d.m, sia ? g_const.sia_m : g_const.b2_m, sizeof d.m);
+  std::memcpy(d.m, sia ? c.sia_m : c.b2_m, sizeof d.m);
   std::memcpy(p.blob, &d, sizeof d);
   p.items = a.threads;
   return HF_OK;
 }
 
-int prepare(KernelId id, const void *args, Prepared &p) {
+// `consts`: the constants a search kernel is launched with; null = the process-wide set as it is now.
+int prepare(KernelId id, const void *args, Prepared &p, const SearchConstants *consts = nullptr) {
   if (!args) return fail(HF_EINVAL, "null argument list");
   p = Prepared();
   p.id = id;
+  SearchConstants process;
+  if (is_crypto(id) && !consts) {
+    process = snapshot_process_constants();
+    consts = &process;
+  }
   switch (id) {
     case K_IM2COL: return prepare_im2col(*static_cast<const hf_im2col_args *>(args), p);
     case K_MAXPOOL: return prepare_maxpool(*static_cast<const hf_maxpool_args *>(args), p);
@@ -451,10 +487,10 @@ int prepare(KernelId id, const void *args, Prepared &p) {
     case K_UPSAMPLE_NEAREST: return prepare_upsample(*static_cast<const hf_upsample_nearest_args *>(args), p);
     case K_HISTC: return prepare_histc(*static_cast<const hf_histc_args *>(args), p);
     case K_UPSAMPLE_BILINEAR: return prepare_bilinear(*static_cast<const hf_upsample_bilinear_args *>(args), p);
-    case K_ETHASH: return prepare_ethash(*static_cast<const hf_ethash_args *>(args), p);
-    case K_SHA256D: return prepare_sha256d(*static_cast<const hf_sha256d_args *>(args), p);
-    case K_SIA_BLAKE2B: return prepare_blake2b(*static_cast<const hf_blake2b_args *>(args), true, p);
-    case K_BLAKE2B: return prepare_blake2b(*static_cast<const hf_blake2b_args *>(args), false, p);
+    case K_ETHASH: return prepare_ethash(*static_cast<const hf_ethash_args *>(args), *consts, p);
+    case K_SHA256D: return prepare_sha256d(*static_cast<const hf_sha256d_args *>(args), *consts, p);
+    case K_SIA_BLAKE2B: return prepare_blake2b(*static_cast<const hf_blake2b_args *>(args), true, *consts, p);
+    case K_BLAKE2B: return prepare_blake2b(*static_cast<const hf_blake2b_args *>(args), false, *consts, p);
     default: return fail(HF_ENOTFOUND, "unknown kernel id");
   }
 }
@@ -482,6 +518,16 @@ unsigned default_grid(const Prepared &p, unsigned own_threads, unsigned block_th
 
 constexpr unsigned kDefaultEthashGrid = 8192;  // the authors' launches: scripts/data/ethminer_event.csv
 
+// A body that counts its work items in 32 bits steps its index past the last item once before the
+// loop test ends it (twice in the exact-2x upsampling path, which takes two items per trip): with
+// `threads` threads striding over `p.items` items the counter reaches items + 2 * threads at most,
+// which must not wrap.  (The searches and the 64-bit paths count in 64 bits.)
+bool counter_fits(const Prepared &p, unsigned long long threads) {
+  return !p.idx32 || p.items + 2ull * threads <= (1ull << 32);
+}
+const char *const kCounterMsg =
+    "work items + 2 * grid_blocks * block threads must fit 32 bits (this path indexes its work items with a 32-bit counter)";
+
 int do_launch_native(KernelId id, const Prepared &p, int grid_blocks, unsigned block, hipStream_t stream) {
   if (block == 0 || block % kWave != 0 || block > (is_crypto(id) ? 512u : kMaxBlock))
     return fail(HF_EINVAL, "block size must be a multiple of 64 within the kernel's launch bound");
@@ -492,6 +538,7 @@ int do_launch_native(KernelId id, const Prepared &p, int grid_blocks, unsigned b
   if (!p.exact_grid && p.items == 0) return HF_OK;  // nothing to do
   if ((unsigned long long)grid * block > 0xFFFFFFFFull)
     return fail(HF_EINVAL, "grid_blocks * block threads must fit 32 bits (the bodies index work items with 32-bit counters)");
+  if (!counter_fits(p, (unsigned long long)grid * block)) return fail(HF_EINVAL, kCounterMsg);
   hipError_t e = is_crypto(id) ? launch_native_crypto(id, p.blob, p.hint, grid, block, p.lds, stream)
                                : launch_native_dl(id, p.blob, p.hint, grid, block, p.lds, stream);
   if (e != hipSuccess) return hip_fail(e, "native launch");
@@ -505,7 +552,13 @@ struct hf_config {
   Config cfg;
 };
 
+struct hf_constants {
+  SearchConstants c;
+};
+
 struct hf_plan {
+  bool has_consts = false;             // hf_plan_bind_constants: launches of this plan use `consts`
+  SearchConstants consts;
   KernelRow rows[2];
   KernelId ids[2];
   const Preset *preset;
@@ -804,16 +857,50 @@ HF_API int hf_plan_local_index(const hf_plan *plan, int half, uint32_t tid, hf_d
 }
 
 // ------------------------------------------------------------- constants
-HF_API int hf_ethash_set_constants(const void *dag, uint32_t dag_items, const uint8_t header[32], uint64_t target,
-                                   void *) try {
+namespace {
+int store_ethash(SearchConstants &c, const void *dag, uint32_t dag_items, const uint8_t *header, uint64_t target) {
   if (!dag || !header) return fail(HF_EINVAL, "ethash: null dag or header");
   if (dag_items == 0) return fail(HF_EINVAL, "ethash: empty dag");
   if (!aligned16(dag)) return fail(HF_EINVAL, "ethash: dag must be 16-byte aligned");
-  std::lock_guard<std::mutex> lock(g_const.mu);
-  g_const.dag = dag;
-  g_const.dag_items = dag_items;
-  for (int i = 0; i < 4; i++) g_const.eth_header[i] = load_le64(header + 8 * i);
-  g_const.eth_target = target;
+  c.dag = dag;
+  c.dag_items = dag_items;
+  for (int i = 0; i < 4; i++) c.eth_header[i] = load_le64(header + 8 * i);
+  c.eth_target = target;
+  c.eth_set = true;
+  return HF_OK;
+}
+int store_sha256d(SearchConstants &c, const uint8_t *header, uint64_t target64) {
+  if (!header) return fail(HF_EINVAL, "sha256d: null header");
+  uint32_t st[8] = {0x6a09e667, 0xbb67ae85, 0x3c6ef372, 0xa54ff53a, 0x510e527f, 0x9b05688c, 0x1f83d9ab, 0x5be0cd19};
+  uint32_t blk[16];
+  for (int i = 0; i < 16; i++) blk[i] = load_be32(header + 4 * i);
+  host_sha256_compress(st, blk);
+  std::memcpy(c.sha_mid, st, sizeof st);
+  for (int i = 0; i < 3; i++) c.sha_tail[i] = load_be32(header + 64 + 4 * i);
+  c.sha_target = target64;
+  c.sha_set = true;
+  return HF_OK;
+}
+int store_blake2b(SearchConstants &c, bool sia, const uint8_t *header) {
+  if (!header) return fail(HF_EINVAL, sia ? "sia_blake2b: null header" : "blake2b: null header");
+  uint64_t *m = sia ? c.sia_m : c.b2_m;
+  for (int i = 0; i < 10; i++) m[i] = load_le64(header + 8 * i);
+  (sia ? c.sia_set : c.b2_set) = true;
+  return HF_OK;
+}
+}  // namespace
+
+// The process-wide set: each call builds the new values aside and swaps them in under the lock.
+HF_API int hf_ethash_set_constants(const void *dag, uint32_t dag_items, const uint8_t header[32], uint64_t target,
+                                   void *) try {
+  SearchConstants c;
+  int rc = store_ethash(c, dag, dag_items, header, target);
+  if (rc != HF_OK) return rc;
+  std::lock_guard<std::mutex> lock(g_const_mu);
+  g_const.dag = c.dag;
+  g_const.dag_items = c.dag_items;
+  std::memcpy(g_const.eth_header, c.eth_header, sizeof c.eth_header);
+  g_const.eth_target = c.eth_target;
   g_const.eth_set = true;
   return HF_OK;
 } catch (...) {
@@ -821,15 +908,13 @@ HF_API int hf_ethash_set_constants(const void *dag, uint32_t dag_items, const ui
 }
 
 HF_API int hf_sha256d_set_block(const uint8_t header[80], uint64_t target64, void *) try {
-  if (!header) return fail(HF_EINVAL, "sha256d: null header");
-  uint32_t st[8] = {0x6a09e667, 0xbb67ae85, 0x3c6ef372, 0xa54ff53a, 0x510e527f, 0x9b05688c, 0x1f83d9ab, 0x5be0cd19};
-  uint32_t blk[16];
-  for (int i = 0; i < 16; i++) blk[i] = load_be32(header + 4 * i);
-  host_sha256_compress(st, blk);
-  std::lock_guard<std::mutex> lock(g_const.mu);
-  std::memcpy(g_const.sha_mid, st, sizeof st);
-  for (int i = 0; i < 3; i++) g_const.sha_tail[i] = load_be32(header + 64 + 4 * i);
-  g_const.sha_target = target64;
+  SearchConstants c;
+  int rc = store_sha256d(c, header, target64);
+  if (rc != HF_OK) return rc;
+  std::lock_guard<std::mutex> lock(g_const_mu);
+  std::memcpy(g_const.sha_mid, c.sha_mid, sizeof c.sha_mid);
+  std::memcpy(g_const.sha_tail, c.sha_tail, sizeof c.sha_tail);
+  g_const.sha_target = c.sha_target;
   g_const.sha_set = true;
   return HF_OK;
 } catch (...) {
@@ -837,9 +922,11 @@ HF_API int hf_sha256d_set_block(const uint8_t header[80], uint64_t target64, voi
 }
 
 HF_API int hf_sia_blake2b_set_block(const uint8_t header[80], void *) try {
-  if (!header) return fail(HF_EINVAL, "sia_blake2b: null header");
-  std::lock_guard<std::mutex> lock(g_const.mu);
-  for (int i = 0; i < 10; i++) g_const.sia_m[i] = load_le64(header + 8 * i);
+  SearchConstants c;
+  int rc = store_blake2b(c, true, header);
+  if (rc != HF_OK) return rc;
+  std::lock_guard<std::mutex> lock(g_const_mu);
+  std::memcpy(g_const.sia_m, c.sia_m, sizeof c.sia_m);
   g_const.sia_set = true;
   return HF_OK;
 } catch (...) {
@@ -847,28 +934,94 @@ HF_API int hf_sia_blake2b_set_block(const uint8_t header[80], void *) try {
 }
 
 HF_API int hf_blake2b_set_block(const uint8_t header[80], void *) try {
-  if (!header) return fail(HF_EINVAL, "blake2b: null header");
-  std::lock_guard<std::mutex> lock(g_const.mu);
-  for (int i = 0; i < 10; i++) g_const.b2_m[i] = load_le64(header + 8 * i);
+  SearchConstants c;
+  int rc = store_blake2b(c, false, header);
+  if (rc != HF_OK) return rc;
+  std::lock_guard<std::mutex> lock(g_const_mu);
+  std::memcpy(g_const.b2_m, c.b2_m, sizeof c.b2_m);
   g_const.b2_set = true;
   return HF_OK;
 } catch (...) {
   return trap_exception();
 }
 
+// Caller-owned sets.
+HF_API int hf_constants_create(hf_constants **out) try {
+  if (!out) return fail(HF_EINVAL, "null output pointer");
+  *out = new hf_constants();
+  return HF_OK;
+} catch (...) {
+  return trap_exception();
+}
+
+HF_API void hf_constants_free(hf_constants *c) { delete c; }
+
+HF_API int hf_constants_set_ethash(hf_constants *c, const void *dag, uint32_t dag_items, const uint8_t header[32],
+                                   uint64_t target) try {
+  if (!c) return fail(HF_EINVAL, "null constants");
+  return store_ethash(c->c, dag, dag_items, header, target);
+} catch (...) {
+  return trap_exception();
+}
+
+HF_API int hf_constants_set_sha256d(hf_constants *c, const uint8_t header[80], uint64_t target64) try {
+  if (!c) return fail(HF_EINVAL, "null constants");
+  return store_sha256d(c->c, header, target64);
+} catch (...) {
+  return trap_exception();
+}
+
+HF_API int hf_constants_set_sia_blake2b(hf_constants *c, const uint8_t header[80]) try {
+  if (!c) return fail(HF_EINVAL, "null constants");
+  return store_blake2b(c->c, true, header);
+} catch (...) {
+  return trap_exception();
+}
+
+HF_API int hf_constants_set_blake2b(hf_constants *c, const uint8_t header[80]) try {
+  if (!c) return fail(HF_EINVAL, "null constants");
+  return store_blake2b(c->c, false, header);
+} catch (...) {
+  return trap_exception();
+}
+
+HF_API int hf_plan_bind_constants(hf_plan *plan, const hf_constants *c) try {
+  if (!plan) return fail(HF_EINVAL, "null plan");
+  plan->has_consts = c != nullptr;
+  if (c) plan->consts = c->c;
+  return HF_OK;
+} catch (...) {
+  return trap_exception();
+}
+
 // ---------------------------------------------------------------- launches
-HF_API int hf_launch_native(const char *kernel_name, const void *args, int grid_blocks, int block_threads,
-                            void *stream) try {
+namespace {
+int launch_native_named(const char *kernel_name, const void *args, const SearchConstants *consts, int grid_blocks,
+                        int block_threads, void *stream) {
   if (!kernel_name) return fail(HF_EINVAL, "null kernel name");
   KernelId id;
   if (!lookup_kernel(kernel_name, id))
     return fail(HF_ENOTFOUND, std::string("kernel '") + kernel_name + "' has no gfx950 implementation in this library");
   Prepared p;
-  int rc = prepare(id, args, p);
+  int rc = prepare(id, args, p, consts);
   if (rc != HF_OK) return rc;
   unsigned block = block_threads > 0 ? (unsigned)block_threads
                                      : (is_crypto(id) ? 128u : (id == K_MAXPOOL ? 256u : (id == K_HISTC ? 768u : 512u)));
   return do_launch_native(id, p, grid_blocks, block, static_cast<hipStream_t>(stream));
+}
+}  // namespace
+
+HF_API int hf_launch_native(const char *kernel_name, const void *args, int grid_blocks, int block_threads,
+                            void *stream) try {
+  return launch_native_named(kernel_name, args, nullptr, grid_blocks, block_threads, stream);
+} catch (...) {
+  return trap_exception();
+}
+
+HF_API int hf_launch_native_with(const char *kernel_name, const void *args, const hf_constants *constants,
+                                 int grid_blocks, int block_threads, void *stream) try {
+  if (!constants) return fail(HF_EINVAL, "null constants");
+  return launch_native_named(kernel_name, args, &constants->c, grid_blocks, block_threads, stream);
 } catch (...) {
   return trap_exception();
 }
@@ -896,6 +1049,11 @@ int do_launch_fused(const hf_plan *plan, const Prepared &p1, const Prepared &p2,
                            ? plan->bounded != 0
                            : plan->preset->launch_bound &&
                                  (unsigned long long)plan->part.launch_blocks * plan->part.launch_threads > 4ull * 256ull;
+  // every thread of the launch may run either body (lending), so each 32-bit counter is checked against all of them
+  auto counters_fit = [&](unsigned grid, unsigned block) {
+    const unsigned long long threads = (unsigned long long)grid * block;
+    return threads <= 0xFFFFFFFFull && counter_fits(p1, threads) && counter_fits(p2, threads);
+  };
   hipError_t e;
   if (plan->preset->base_line) {
     // Vertical baseline: both kernels start at thread 0 of a block of max(d1, d2) threads.
@@ -904,6 +1062,7 @@ int do_launch_fused(const hf_plan *plan, const Prepared &p1, const Prepared &p2,
     g.grid2 = p2.exact_grid ? exact : (grid_blocks > 0 ? (unsigned)grid_blocks : default_grid(p2, g.d2, block));
     const size_t lds = 4 * kBarrierWords + g.lds1 + g.lds2;
     const unsigned grid = std::max(g.grid1, g.grid2);
+    if (!counters_fit(grid, block)) return fail(HF_EINVAL, kCounterMsg);
     e = crypto ? launch_fused_crypto(plan->ids[0], plan->ids[1], MODE_VERTICAL, bounded, p1.blob, p2.blob, g, grid, lds, stream)
                : launch_fused_dl(plan->ids[0], plan->ids[1], MODE_VERTICAL, bounded, p1.blob, p2.blob, g, grid, lds, stream);
   } else if (plan->barrier_mode == HF_BARRIER_BLOCKIDX) {
@@ -916,6 +1075,8 @@ int do_launch_fused(const hf_plan *plan, const Prepared &p1, const Prepared &p2,
       g.grid2 = std::max(1u, (unsigned)grid_blocks - g.grid1);
     }
     const size_t lds = std::max(g.lds1, g.lds2);
+    if ((unsigned long long)g.grid1 + g.grid2 > 0xFFFFFFFFull || !counters_fit(g.grid1 + g.grid2, block))
+      return fail(HF_EINVAL, kCounterMsg);
     e = crypto ? launch_fused_crypto(plan->ids[0], plan->ids[1], MODE_BLOCKIDX, false, p1.blob, p2.blob, g, g.grid1 + g.grid2, lds, stream)
                : launch_fused_dl(plan->ids[0], plan->ids[1], MODE_BLOCKIDX, false, p1.blob, p2.blob, g, g.grid1 + g.grid2, lds, stream);
   } else {
@@ -942,6 +1103,7 @@ int do_launch_fused(const hf_plan *plan, const Prepared &p1, const Prepared &p2,
         g.grid1 = g.grid2 + (unsigned)(((unsigned long long)(g.grid1 - g.grid2) * g.d1 + dd - 1) / dd);
     }
     const unsigned grid = std::max(g.grid1, g.grid2);
+    if (!counters_fit(grid, block)) return fail(HF_EINVAL, kCounterMsg);
     const size_t lds = 4 * kBarrierWords + g.lds1 + g.lds2;
     const FuseMode mode = plan->barrier_mode == HF_BARRIER_MATCHED ? MODE_MATCHED : MODE_HFUSE;
     e = crypto ? launch_fused_crypto(plan->ids[0], plan->ids[1], mode, bounded, p1.blob, p2.blob, g, grid, lds, stream)
@@ -957,9 +1119,10 @@ int do_launch_fused(const hf_plan *plan, const Prepared &p1, const Prepared &p2,
 HF_API int hf_launch_fused(const hf_plan *plan, const void *args1, const void *args2, int grid_blocks, void *stream) try {
   if (!plan) return fail(HF_EINVAL, "null plan");
   Prepared p1, p2;
-  int rc = prepare(plan->ids[0], args1, p1);
+  const SearchConstants *consts = plan->has_consts ? &plan->consts : nullptr;
+  int rc = prepare(plan->ids[0], args1, p1, consts);
   if (rc != HF_OK) return rc;
-  rc = prepare(plan->ids[1], args2, p2);
+  rc = prepare(plan->ids[1], args2, p2, consts);
   if (rc != HF_OK) return rc;
   return do_launch_fused(plan, p1, p2, grid_blocks, static_cast<hipStream_t>(stream));
 } catch (...) {
@@ -990,10 +1153,11 @@ HF_API int hf_time_pair(const hf_plan *plan, int mode, const void *const *args1,
     if (se != hipSuccess) return hip_fail(se, "second stream");
   }
   std::vector<Prepared> p1(nsets), p2(nsets);
+  const SearchConstants *consts = plan->has_consts ? &plan->consts : nullptr;
   for (int i = 0; i < nsets; i++) {
-    int rc = prepare(plan->ids[0], args1[i], p1[i]);
+    int rc = prepare(plan->ids[0], args1[i], p1[i], consts);
     if (rc != HF_OK) return rc;
-    rc = prepare(plan->ids[1], args2[i], p2[i]);
+    rc = prepare(plan->ids[1], args2[i], p2[i], consts);
     if (rc != HF_OK) return rc;
   }
   const unsigned b1 = plan->rows[0].native_block(), b2 = plan->rows[1].native_block();

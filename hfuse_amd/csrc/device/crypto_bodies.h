@@ -99,9 +99,10 @@ struct Sha256dBody {
 
   template <class SB>
   static __device__ __forceinline__ void run(const Args &a, SB &sb, unsigned char *, unsigned) {
-    const u32 stride = sb.gstride();
-    for (u32 t = sb.gtid(); t < a.threads; t += stride) {
-      const u32 nonce = a.start_nonce + t;
+    // 64-bit counter: `threads` may be anything up to 2^32 - 1, so t + stride must not wrap
+    const u64 stride = sb.gstride();
+    for (u64 t = sb.gtid(); t < a.threads; t += stride) {
+      const u32 nonce = a.start_nonce + (u32)t;
       u32 st[8], w[16];
 #pragma unroll
       for (int i = 0; i < 8; i++) st[i] = a.midstate[i];
@@ -225,9 +226,9 @@ struct Blake2bBody {
 
   template <class SB>
   static __device__ __forceinline__ void run(const Args &a, SB &sb, unsigned char *, unsigned) {
-    const u32 stride = sb.gstride();
-    for (u32 t = sb.gtid(); t < a.threads; t += stride) {
-      const u32 nonce = a.start_nonce + t;
+    const u64 stride = sb.gstride();  // 64-bit counter: t + stride must not wrap for any `threads`
+    for (u64 t = sb.gtid(); t < a.threads; t += stride) {
+      const u32 nonce = a.start_nonce + (u32)t;
       u64 m[16], v[16];
 #pragma unroll
       for (int i = 0; i < 10; i++) m[i] = a.m[i];

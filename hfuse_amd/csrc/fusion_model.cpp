@@ -277,6 +277,13 @@ int make_partition(const KernelRow &k1, const KernelRow &k2, const Preset &prese
   } else {
     variant += "_idx_0";  // main.cpp:218-219,223: the vertical presets print one variant
     if (std::max(dims[0].size(), dims[1].size()) > kMaxBlock) { err = "block exceeds 1024 threads"; return HF_EINVAL; }
+    // the vertical kernel hands each body whole wavefronts too: a ragged BlockDim would leave its last lanes' items undone
+    for (int i = 0; i < 2; i++) {
+      if (dims[i].size() % kWave != 0) {
+        err = "BlockDim of '" + rows[i]->name + "' is " + std::to_string(dims[i].size()) + " threads: not a multiple of the 64-lane wavefront";
+        return HF_EINVAL;
+      }
+    }
   }
 
   uint32_t b = 0;

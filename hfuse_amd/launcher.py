@@ -129,6 +129,10 @@ class Plan:
         """True / False: run the register-bounded / the plain build; None: by the preset."""
         check(L.lib().hf_plan_set_launch_bound(self._h, -1 if on is None else int(bool(on))))
 
+    def bind_constants(self, constants: Optional["Constants"]) -> None:
+        """Fused launches of this plan use a copy of `constants` instead of the process-wide set (None unbinds)."""
+        check(L.lib().hf_plan_bind_constants(self._h, constants._h if constants is not None else None))
+
     def local_index(self, half: int, tid: int):
         out = L.Dim3()
         check(L.lib().hf_plan_local_index(self._h, half, tid, C.byref(out)))
@@ -151,9 +155,49 @@ class Plan:
         return ms.value
 
 
-def launch_native(kernel_name: str, args, grid_blocks: int = 0, block_threads: int = 0, stream=None) -> None:
+def launch_native(kernel_name: str, args, grid_blocks: int = 0, block_threads: int = 0, stream=None,
+                  constants: Optional["Constants"] = None) -> None:
+    if constants is not None:
+        check(L.lib().hf_launch_native_with(kernel_name.encode(), C.byref(args), constants._h, grid_blocks,
+                                            block_threads, _stream_ptr(stream)))
+        return
     check(L.lib().hf_launch_native(kernel_name.encode(), C.byref(args), grid_blocks, block_threads,
                                    _stream_ptr(stream)))
+
+
+class Constants:
+    """A caller-owned set of the search kernels' constants (DAG, headers, targets): one per host thread or job."""
+
+    def __init__(self):
+        self._h = C.c_void_p()
+        self._keep = []
+        check(L.lib().hf_constants_create(C.byref(self._h)))
+
+    def __del__(self):
+        if getattr(self, "_h", None) and L is not None and L._lib is not None:
+            L._lib.hf_constants_free(self._h)
+            self._h = None
+
+    def set_ethash(self, dag, dag_items: int, header: bytes, target: int) -> "Constants":
+        assert len(header) == 32
+        self._keep = [dag]
+        check(L.lib().hf_constants_set_ethash(self._h, C.c_void_p(dag.data_ptr()), dag_items, header, target))
+        return self
+
+    def set_sha256d(self, header: bytes, target64: int) -> "Constants":
+        assert len(header) == 80
+        check(L.lib().hf_constants_set_sha256d(self._h, header, target64))
+        return self
+
+    def set_sia_blake2b(self, header: bytes) -> "Constants":
+        assert len(header) == 80
+        check(L.lib().hf_constants_set_sia_blake2b(self._h, header))
+        return self
+
+    def set_blake2b(self, header: bytes) -> "Constants":
+        assert len(header) == 80
+        check(L.lib().hf_constants_set_blake2b(self._h, header))
+        return self
 
 
 # ------------------------------------------------------------ argument builders

@@ -151,7 +151,9 @@ def splitmix64_bytes(n: int, seed: int) -> bytes:
 class SearchPair:
     """Two nonce searches with their constants uploaded: `fresh()` -> (results1, results2, args1, args2).
 
-    Constants are per process (hf_*_set_block), so only one SearchPair is live at a time.
+    The constants live in `self.constants` (a caller-owned set: bind it to a plan with
+    `plan.bind_constants(pair.constants)` or pass it to `launch_native`); they are also written to the
+    process-wide set, which the split tuner's own plans read, so one SearchPair at a time there.
     `grid` is the grid a native Ethash launch of 128-thread blocks needs for its nonce count (Ethash
     scans gridDim * blockDim nonces); a fused launch divides by Ethash's share of the block instead."""
 
@@ -168,6 +170,7 @@ class SearchPair:
         self.dag_items = dag_items
         self._keep = []
         self.grid = 0
+        self.constants = H.Constants()
         for pos, k in enumerate((k1, k2)):
             hdr = splitmix64_bytes(32 if k == "ethash_search" else 80, SEED + 100 + pos)
             self.headers.append(hdr)
@@ -176,15 +179,19 @@ class SearchPair:
                 H.fill_splitmix64(dag, SEED)
                 torch.cuda.synchronize()
                 H.ethash_set_constants(dag, dag_items, hdr, self.ETHASH_TARGET)
+                self.constants.set_ethash(dag, dag_items, hdr, self.ETHASH_TARGET)
                 self._keep.append(dag)
                 if pos == 0:
                     self.grid = self.nonces[0] // 128
             elif k == "sha256d_gpu_hash_shared":
                 H.sha256d_set_block(hdr, self.TARGET32)
+                self.constants.set_sha256d(hdr, self.TARGET32)
             elif k == "sia_blake2b_gpu_hash":
                 H.sia_blake2b_set_block(hdr)
+                self.constants.set_sia_blake2b(hdr)
             elif k == "blake2b_gpu_hash":
                 H.blake2b_set_block(hdr)
+                self.constants.set_blake2b(hdr)
             else:
                 raise KeyError(k)
 

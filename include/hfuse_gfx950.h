@@ -355,8 +355,16 @@ typedef struct {
 
 /*
  * Constants the original kernels read from __constant__ symbols set by their
- * host program.  Each call copies to this library's own device symbols on
- * `stream`; they hold until the next call.
+ * host program (DAG pointer and size, header, midstate, target).  The library
+ * keeps them in host memory and passes them in the kernel-argument segment of
+ * each launch, next to the original argument list; nothing is copied to the
+ * device by these calls and `stream` is ignored (kept for source compatibility
+ * with a cudaMemcpyToSymbolAsync-style caller).
+ *
+ * These four calls write ONE process-wide set, as the original symbols are one
+ * per device: each call replaces its values atomically, and every launch reads
+ * the set as it is when the launch call is made.  Two host threads that search
+ * different headers must not share it -- they use hf_constants below.
  */
 /* ethash: DAG of 128-byte items, 32-byte header hash, 64-bit target. */
 HF_API int hf_ethash_set_constants(const void *dag, uint32_t dag_items, const uint8_t header[32],
@@ -368,6 +376,23 @@ HF_API int hf_sha256d_set_block(const uint8_t header[80], uint64_t target64, voi
 HF_API int hf_sia_blake2b_set_block(const uint8_t header[80], void *stream);
 HF_API int hf_blake2b_set_block(const uint8_t header[80], void *stream);
 
+/*
+ * A caller-owned set of the same constants (no counterpart in the reference, whose host
+ * programs are single-threaded).  One thread fills it; hf_plan_bind_constants copies it into
+ * a plan, whose fused launches then use that copy instead of the process-wide set (NULL
+ * unbinds), and hf_launch_native_with launches one original kernel with it.  Setting the
+ * constants and launching is thereby one unit per plan / per call, whatever other threads do.
+ */
+typedef struct hf_constants hf_constants;
+HF_API int hf_constants_create(hf_constants **out);
+HF_API void hf_constants_free(hf_constants *c);
+HF_API int hf_constants_set_ethash(hf_constants *c, const void *dag, uint32_t dag_items,
+                                   const uint8_t header[32], uint64_t target);
+HF_API int hf_constants_set_sha256d(hf_constants *c, const uint8_t header[80], uint64_t target64);
+HF_API int hf_constants_set_sia_blake2b(hf_constants *c, const uint8_t header[80]);
+HF_API int hf_constants_set_blake2b(hf_constants *c, const uint8_t header[80]);
+HF_API int hf_plan_bind_constants(hf_plan *plan, const hf_constants *c);
+
 /* ----------------------------------------------------------------- launches */
 /*
  * Native launch of one original kernel by its YAML name; `args` points at the
@@ -377,6 +402,10 @@ HF_API int hf_blake2b_set_block(const uint8_t header[80], void *stream);
  */
 HF_API int hf_launch_native(const char *kernel_name, const void *args, int grid_blocks,
                             int block_threads, void *stream);
+/* The same with the search constants of `constants` instead of the process-wide set. */
+HF_API int hf_launch_native_with(const char *kernel_name, const void *args,
+                                 const hf_constants *constants, int grid_blocks, int block_threads,
+                                 void *stream);
 /*
  * Fused launch: one kernel whose workgroup is [0,d1) running kernel 1's body
  * and [d1,d1+d2) running kernel 2's, arguments in YAML order

@@ -429,6 +429,96 @@ def test_launch_argument_errors_never_reach_the_gpu(cfg):
     assert b"32 bits" in lib.hf_last_error()
 
 
+def test_counter_wrap_is_refused_on_the_host(cfg):
+    """A caller grid large enough that a 32-bit work-item counter would wrap (and never end its loop)
+    is refused; the searches count in 64 bits, so a full-range scan (threads = 2^32 - 1) passes the
+    validators and only fails for want of a device."""
+    lib = L.lib()
+    up = L.UpsampleNearestArgs()
+    up.idata = up.odata = 256
+    up.nc, up.height1, up.width1, up.height2, up.width2 = 1 << 11, 512, 512, 1024, 1024  # 2^28 work items in the exact-2x path
+    up.height_scale = up.width_scale = 0.5
+    # two items per trip: 2^28 + 2 * grid * block must stay within 2^32
+    assert lib.hf_launch_native(b"upsample_nearest2d_out_frame", C.byref(up), 1 << 22, 512, None) == L.HF_EINVAL
+    assert b"32 bits" in lib.hf_last_error()
+    ok = lib.hf_launch_native(b"upsample_nearest2d_out_frame", C.byref(up), 1 << 20, 512, None)
+    assert ok in (L.HF_OK, L.HF_EHIP), lib.hf_last_error()
+    hdr = bytes(range(80))
+    assert lib.hf_sha256d_set_block(hdr, 1, None) == 0 and lib.hf_sia_blake2b_set_block(hdr, None) == 0
+    sh = L.Sha256dArgs()
+    sh.threads, sh.start_nonce, sh.res_nonces = 0xFFFFFFFF, 0, 256
+    b2 = L.Blake2bArgs()
+    b2.threads, b2.start_nonce, b2.res_nonce = 0xFFFFFFFF, 0, 256
+    import torch
+    if not torch.cuda.is_available():   # with a device these would launch on made-up pointers
+        assert lib.hf_launch_native(b"sha256d_gpu_hash_shared", C.byref(sh), 0, 0, None) in (L.HF_OK, L.HF_EHIP)
+        assert lib.hf_launch_native(b"sia_blake2b_gpu_hash", C.byref(b2), 0, 0, None) in (L.HF_OK, L.HF_EHIP)
+
+
+def test_vertical_presets_need_whole_wavefronts():
+    """A BlockDim that is not a multiple of 64 threads is refused under vfuse / vfuse_lb as under hfuse:
+    the vertical kernel runs whole wavefronts of each body and would leave the ragged lanes' items undone."""
+    table = KERNELS_MAP.replace("X: 512", "X: 96", 1)
+    c = Config(FUSION, table)
+    for preset in ("vfuse", "vfuse_lb", "hfuse"):
+        with pytest.raises(hfuse_amd.HfuseError) as e:
+            c.plan(0, preset)
+        assert e.value.code == L.HF_EINVAL and "wavefront" in e.value.message, preset
+
+
+def test_bilinear_scales_are_validated():
+    """Scales that would send the unclamped source index outside the input (too large, inf, NaN) are refused."""
+    lib = L.lib()
+    def args(rh, rw, align=0):
+        bl = L.UpsampleBilinearArgs()
+        bl.n, bl.rheight, bl.rwidth, bl.align_corners = 256, rh, rw, align
+        bl.idata.data = bl.odata.data = 256
+        bl.idata.sizes[:] = [2, 3, 8, 8]; bl.idata.strides[:] = [192, 64, 8, 1]
+        bl.odata.sizes[:] = [2, 3, 16, 16]; bl.odata.strides[:] = [768, 256, 16, 1]
+        return bl
+    for rh, rw, align in ((float("inf"), 0.5, 0), (0.5, float("inf"), 0), (float("nan"), 0.5, 0), (0.6, 0.5, 0),
+                          (0.5, 0.6, 0), (0.5, 8.0 / 15.0 + 1e-3, 1), (1e30, 0.5, 1), (-0.5, 0.5, 0)):
+        a = args(rh, rw, align)
+        assert lib.hf_launch_native(b"upsample_bilinear2d_out_frame", C.byref(a), 0, 0, None) == L.HF_EINVAL, (rh, rw, align)
+    import torch
+    if not torch.cuda.is_available():
+        for rh, rw, align in ((0.5, 0.5, 0), (7.0 / 15.0, 7.0 / 15.0, 1), (0.25, 0.5, 0), (0.0, 0.0, 1)):
+            a = args(rh, rw, align)
+            assert lib.hf_launch_native(b"upsample_bilinear2d_out_frame", C.byref(a), 0, 0, None) in (L.HF_OK, L.HF_EHIP), \
+                (rh, rw, align, lib.hf_last_error())
+
+
+def test_constants_objects_are_independent_of_the_process_wide_set(cfg):
+    """hf_constants: a caller-owned set; a plan bound to it, or hf_launch_native_with, does not look at the
+    process-wide set at all (here the process-wide Ethash constants are unset in a fresh library state
+    only if no other test set them, so the check goes through an unset *caller-owned* set instead)."""
+    lib = L.lib()
+    from hfuse_amd import launcher as H
+    empty, full = H.Constants(), H.Constants()
+    hdr = bytes(range(80))
+    full.set_sha256d(hdr, 1).set_sia_blake2b(hdr)
+    sh = L.Sha256dArgs()
+    sh.threads, sh.start_nonce, sh.res_nonces = 0, 0, 256     # zero nonces: validated, nothing launched
+    assert lib.hf_sha256d_set_block(hdr, 1, None) == 0         # process-wide set has it ...
+    assert lib.hf_launch_native_with(b"sha256d_gpu_hash_shared", C.byref(sh), empty._h, 0, 0, None) == L.HF_EINVAL
+    assert b"hf_sha256d_set_block" in lib.hf_last_error()      # ... the empty caller-owned set does not
+    assert lib.hf_launch_native_with(b"sha256d_gpu_hash_shared", C.byref(sh), full._h, 0, 0, None) == L.HF_OK
+    assert lib.hf_launch_native_with(b"sha256d_gpu_hash_shared", C.byref(sh), None, 0, 0, None) == L.HF_EINVAL
+    i = cfg.find_fusion("sha256d_gpu_hash_shared", "sia_blake2b_gpu_hash")
+    plan = cfg.plan(i)
+    b2 = L.Blake2bArgs()
+    b2.threads, b2.start_nonce, b2.res_nonce = 0, 0, 256
+    plan.bind_constants(empty)
+    assert lib.hf_launch_fused(plan._h, C.byref(sh), C.byref(b2), 0, None) == L.HF_EINVAL
+    plan.bind_constants(None)                                  # back to the process-wide set
+    assert lib.hf_sia_blake2b_set_block(hdr, None) == 0
+    import torch
+    if not torch.cuda.is_available():
+        assert lib.hf_launch_fused(plan._h, C.byref(sh), C.byref(b2), 0, None) in (L.HF_OK, L.HF_EHIP)
+    with pytest.raises(hfuse_amd.HfuseError):
+        H.Constants().set_ethash(type("T", (), {"data_ptr": lambda self: 8})(), 4, bytes(32), 1)  # misaligned DAG
+
+
 def test_header_symbols_are_all_exported():
     """Every function include/hfuse_gfx950.h declares is exported by the built library."""
     import os
@@ -505,7 +595,13 @@ def test_partition_matches_oracle_on_random_kernel_tables():
                 checked += 1
         for preset, lb in (("vfuse", False), ("vfuse_lb", True)):
             want = O.context(rows, base_line=True, launch_bound=lb, imbalanced=False, granule=64, reg_file=4 * 512 * 64, max_threads=2048)
-            got = cfg.plan(0, preset, 0).partition
+            try:
+                got = cfg.plan(0, preset, 0).partition
+            except hfuse_amd.HfuseError as e:   # the vertical kernel runs whole wavefronts of each body too
+                assert e.code == L.HF_EINVAL and any((r[0][0] * r[0][1]) % 64 for r in rows), rows
+                refused += 1
+                continue
+            assert not any((r[0][0] * r[0][1]) % 64 for r in rows), rows
             assert list(got.lo) == [0, 0] == list(want.lo) and list(got.hi) == list(want.hi)
             assert got.launch_threads == want.launch_threads and got.launch_blocks == want.launch_blocks
             checked += 1
