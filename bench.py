@@ -1,23 +1,36 @@
 #!/usr/bin/env python3
 """Benchmark of the five horizontally fused pairs on one MI355X.
 
-A "step" is one launch of the fused kernel of the headline pair (batch-norm
-collect-statistics + upsample_nearest2d at its full shape) over one set of
-synthetic inputs already resident in HBM.  For every pair the script also times
-the two native kernels alone and back to back on one stream, so the metric of
-the reference (fused time vs. the two native launches) can be read per pair.
+A "step" is one launch of the fused kernel of the headline pair -- Ethash over a 4 GiB synthetic
+DAG (2^28 nonces) + Sia-Blake2b (2^30 nonces), the largest of the five benchmark configurations --
+with the DAG, headers and result buffers already resident in HBM.  The timed region is exactly
+`--steps` such launches between two synchronisations.  For every pair the script also times the
+two native kernels alone, back to back on one stream and on two streams, the vertical baseline
+and the register-bounded build, so the metric of the reference (fused time against the two
+native launches) and the three-way native / vertical / horizontal comparison can be read per pair.
+None of these per-pair figures depends on `--steps`: the tensor pairs take at least two full
+rotations of their buffer sets per sample, continuing the rotation from call to call, so no timed
+launch reads inputs that still sit in the 256 MB memory-side cache.
 
 Prints ONE JSON line.  `value` is the headline pair's speedup in percent,
-(t_back_to_back / t_fused - 1) * 100; `pairs` carries the same plus absolute
-GB/s or MH/s and roofline fractions for all five pairs; `roofline` is the
-headline pair's fused kernel against HBM peak; `cpu_baseline` is the CPU oracle
-timed on this host's cores on a bounded sample.
+(t_back_to_back / t_fused - 1) * 100; `pairs` carries the same plus absolute GB/s or MH/s and
+roofline fractions for all five pairs; `roofline` is the headline fused kernel's DAG reads against
+HBM peak; `cpu_baseline` is the CPU restatement of the same two searches timed on this host's cores
+on a bounded sample (and, per tensor pair, PyTorch's CPU operators).
+
+What was timed is also checked: after timing, every tensor pair runs once more on one of its
+rotating sets and the outputs are compared with PyTorch's CPU operators; the searches' fused
+found sets are compared with the native kernels' and every SHA-256d / Blake2b hit is re-hashed
+with hashlib; in the CPU leg the CPU restatement scans the first part of the Ethash and Blake2b
+ranges and its found set must equal the GPU's there.
 """
 from __future__ import annotations
 
 import argparse
+import hashlib
 import json
 import os
+import statistics
 import sys
 import time
 
@@ -26,40 +39,49 @@ sys.path.insert(0, ROOT)
 
 HBM_PEAK_GBPS = 8000.0            # MI355X HBM3E
 VALU_PEAK_GOPS = 256 * 128 * 2.4  # 256 CUs x 128 lanes x 2.4 GHz int32 op/s in Gop/s (= 157.3 TFLOP/s fp32 / 2)
-# HBM bytes per launch of the headline fused kernel from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE, each
-# scaled by what the same counter reads for the plain copy kernel (profiles/tensor_pairs_hbm_traffic.md)
-HEADLINE_TRAFFIC_BYTES = {"bn_upsample": 156.98e6, "im2col_maxpool": 443.28e6, "histc_maxpool": 329.49e6}
+# HBM bytes per launch of each fused kernel from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE, each scaled by what
+# the same counter reads for the plain copy kernel (profiles/tensor_pairs_hbm_traffic.md,
+# profiles/search_pairs_hbm_traffic.md); None where no counter run covers the shape
+TRAFFIC_BYTES = {"bn_upsample": 156.98e6, "im2col_maxpool": 443.28e6, "histc_maxpool": 329.49e6,
+                 "ethash_blake2b": None}
 
 # textbook primitive-op counts per hash (add / logic / rotate / shift = 1 each)
 OPS_SHA256D = 4336
 OPS_BLAKE2B = 2528
 ETHASH_BYTES = 8192               # 64 accesses x 128 bytes of DAG per hash
 
+TENSOR_NAMES = ("im2col_maxpool", "bn_upsample", "histc_maxpool")
+SEARCH_NAMES = ("sha256d_blake2b", "ethash_blake2b")
+MODE_KEYS = {0: "t_a_ms", 1: "t_b_ms", 2: "t_b2b_ms", 3: "t_fused_ms", 4: "t_two_streams_ms"}
+
 
 def parse():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
-    ap.add_argument("--steps", type=int, default=200)
-    ap.add_argument("--warmup", type=int, default=20)
+    ap.add_argument("--steps", type=int, default=10, help="timed launches of the headline fused kernel")
+    ap.add_argument("--warmup", type=int, default=2)
     ap.add_argument("--pairs", default="all", help="comma list of pair names, or 'all'")
-    ap.add_argument("--headline", default="bn_upsample")
+    ap.add_argument("--headline", default="ethash_blake2b")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--sweep", action="store_true",
                     help="also time every split of the reference's enumeration and report the fastest "
                          "(default: the tuned split of the shipped fusion list)")
     ap.add_argument("--fused-only", action="store_true", help="launch only the fused kernel (profiling runs)")
-    ap.add_argument("--search-log2", type=int, default=None, help="override log2 of the nonce ranges (debug)")
+    ap.add_argument("--search-log2", type=int, default=None, help="override log2 of the nonce ranges (profiling runs)")
     ap.add_argument("--extra-pairs", action="store_true",
                     help="also time the other tensor pairs of the shipped fusion list (the reference's ml_fusion.yaml)")
     ap.add_argument("--read-footprint-mb", type=int, default=0,
                     help="MB the smaller read stream of a tensor pair cycles through before a buffer set repeats "
                          "(default 600; below about 300 the memory-side cache serves the reads; at least three sets in any case)")
+    ap.add_argument("--rotations", type=int, default=2,
+                    help="full rotations of a tensor pair's buffer sets per timing sample (launch floor, independent of --steps)")
     ap.add_argument("--calibrate-copy", type=int, default=0, metavar="MIB",
                     help="also run the plain copy kernel on MIB mebibytes (the unit HBM counters are scaled by)")
     return ap.parse_args()
 
 
-from hfuse_amd.workloads import SEED, BENCH_TENSOR_PAIRS, TENSOR_KERNELS, build_pair, build_tensor_pairs  # noqa: E402
+from hfuse_amd.workloads import (SEED, BENCH_TENSOR_PAIRS, TENSOR_KERNELS, SearchPair, build_pair,  # noqa: E402
+                                 build_tensor_pairs)
 
 
 def candidate_plans(cfg, k1, k2, sweep):
@@ -74,44 +96,50 @@ def candidate_plans(cfg, k1, k2, sweep):
     return out
 
 
-def time_tensor_pair(cfg, pair, steps, warmup, sweep, fused_only, rounds=5):
-    """-> dict with per-launch milliseconds of native A, native B, back-to-back and the fused kernel.
+def judge(res):
+    """Adds speedup, the fastest way to run the pair and horizontal-vs-vertical to a per-pair result."""
+    res["speedup_pct"] = (res["t_b2b_ms"] / res["t_fused_ms"] - 1.0) * 100.0
+    ways = {"back_to_back": res["t_b2b_ms"], "two_streams": res["t_two_streams_ms"], "vfuse": res["t_vfuse_ms"],
+            "hfuse": res["t_fused_ms"], "hfuse_lb": res["t_fused_lb_ms"]}
+    res["best_mode"] = min(ways, key=ways.get)
+    res["hfuse_vs_vfuse_pct"] = (res["t_vfuse_ms"] / res["t_fused_ms"] - 1.0) * 100.0
+    res["hfuse_vs_two_streams_pct"] = (res["t_two_streams_ms"] / res["t_fused_ms"] - 1.0) * 100.0
 
-    The four modes are timed in `rounds` interleaved rounds of steps/rounds launches each and the
-    median round is reported, so slow drifts of clocks hit all modes alike."""
-    import statistics
+
+# ------------------------------------------------------------------ tensor pairs
+def time_tensor_pair(cfg, pair, rotations, sweep, fused_only, rounds=5):
+    """-> dict with per-launch milliseconds of native A, native B, back to back, two streams, the vertical
+    baseline, the fused kernel and its register-bounded build.
+
+    Every sample is `rotations` full cycles through the pair's buffer sets (whatever --steps says), each
+    call continues the rotation where the previous one stopped, and the modes are interleaved in
+    `rounds` rounds whose median is reported, so slow drifts of the clocks hit all modes alike."""
+    i = cfg.find_fusion(pair.k1, pair.k2)
     plans = candidate_plans(cfg, pair.k1, pair.k2, sweep)
+    nsets = len(pair.sets)
+    per = max(1, rotations) * nsets
     plan, label = plans[0][1], plans[0][0]
     if len(plans) > 1:
         best = None
-        probe = max(20, steps // 4)
         for lab, p in plans:
-            t = p.time(3, pair.args1, pair.args2, max(5, warmup // 2), probe) / probe
+            t = pair.time(p, 3, 3, per) / per
             if best is None or t < best[0]:
                 best = (t, lab, p)
         _, label, plan = best
-    per = max(1, steps // rounds)
-    modes = [3] if fused_only else [0, 1, 2, 3]
-    samples = {m: [] for m in modes}
-    for r in range(rounds):
-        for m in modes:
-            samples[m].append(plan.time(m, pair.args1, pair.args2, warmup if r == 0 else 2, per) / per)
-    res = {}
-    names = {0: "t_a_ms", 1: "t_b_ms", 2: "t_b2b_ms", 3: "t_fused_ms"}
-    for m in modes:
-        res[names[m]] = statistics.median(samples[m])
+    runs = [("t_fused_ms", plan, 3)]
     if not fused_only:
-        # the reference's vertical baseline (same threads run both bodies), for the three-way comparison
-        vplan = cfg.plan(cfg.find_fusion(pair.k1, pair.k2), "vfuse")
-        res["t_vfuse_ms"] = statistics.median(
-            [vplan.time(3, pair.args1, pair.args2, 2, per) / per for _ in range(3)])
-        # the two natives on two streams at once, the launch pattern of the reference's own traces
-        res["t_two_streams_ms"] = statistics.median(
-            [plan.time(4, pair.args1, pair.args2, 2, per) / per for _ in range(3)])
-        # the launch-bound preset: the same block shape, the build compiled for 8 waves per SIMD
-        lbplan = cfg.plan(cfg.find_fusion(pair.k1, pair.k2), "hfuse_lb")
-        res["t_fused_lb_ms"] = statistics.median(
-            [lbplan.time(3, pair.args1, pair.args2, 2, per) / per for _ in range(3)])
+        runs = [("t_a_ms", plan, 0), ("t_b_ms", plan, 1), ("t_b2b_ms", plan, 2), ("t_fused_ms", plan, 3),
+                ("t_two_streams_ms", plan, 4),                     # the launch pattern of the reference's own traces
+                ("t_vfuse_ms", cfg.plan(i, "vfuse"), 3),           # the reference's vertical baseline
+                ("t_fused_lb_ms", cfg.plan(i, "hfuse_lb"), 3)]     # the same block shape, register-bounded build
+    for _, p, m in runs:                                            # one untimed rotation per mode
+        pair.time(p, m, 0, nsets)
+    samples = {k: [] for k, _, _ in runs}
+    for _ in range(rounds):
+        for key, p, m in runs:
+            samples[key].append(pair.time(p, m, 2, per) / per)
+    res = {k: statistics.median(v) for k, v in samples.items()}
+    res["launches_per_sample"], res["rounds"], res["buffer_sets"] = per, rounds, nsets
     res["split"] = label
     part = plan.partition
     res["fused_name"] = part.name.decode()
@@ -120,59 +148,82 @@ def time_tensor_pair(cfg, pair, steps, warmup, sweep, fused_only, rounds=5):
     return res
 
 
-# ------------------------------------------------------------------ searches
-def time_events(fn, iters):
+def check_tensor_pair(name, pair, plan):
+    """One fused launch on a buffer set the timing rotated through, outputs against PyTorch's CPU operators."""
     import torch
-    a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    F = torch.nn.functional
+    s = len(pair.sets) // 2
+    keep1, keep2 = pair.sets[s]["keep"]
+    if name == "histc_maxpool":
+        keep1[1].zero_()                      # counts accumulate over launches
+    plan.launch(pair.args1[s], pair.args2[s])
     torch.cuda.synchronize()
-    a.record()
-    for _ in range(iters):
-        fn()
-    b.record()
-    b.synchronize()
-    return a.elapsed_time(b) / iters
+
+    def same(got, want, what):
+        assert torch.equal(got.cpu().reshape(want.shape), want), f"{name}: {what} differs from PyTorch CPU"
+
+    def pool(keep, k, st, p):
+        y, val, idx = keep
+        wv, wi = F.max_pool2d(y.cpu(), k, st, p, return_indices=True)
+        same(val, wv, "max_pool2d values")
+        same(idx, wi, "max_pool2d indices")
+
+    if name == "im2col_maxpool":
+        x, col = keep1
+        same(col, F.unfold(x.cpu(), 3, padding=1, stride=1), "im2col")
+        pool(keep2, 3, 2, 1)
+    elif name == "bn_upsample":
+        x, mean, inv = keep1
+        xd = x.cpu().double()
+        wm = xd.mean(dim=(0, 2, 3))
+        wi = 1.0 / torch.sqrt(xd.var(dim=(0, 2, 3), unbiased=False) + 1e-5)
+        for got, want, what in ((mean, wm, "mean"), (inv, wi, "invstd")):
+            err = float(((got.cpu().double() - want).abs() / want.abs().clamp_min(1e-30)).max())
+            assert err <= 1e-5, f"{name}: batch-norm {what} off by {err:.2e} relative (tolerance 1e-5)"
+        u, out = keep2
+        same(out, F.interpolate(u.cpu(), scale_factor=2, mode="nearest"), "upsample_nearest2d")
+    else:
+        x, hist = keep1
+        same(hist, torch.histc(x.cpu(), 1024, 0, 1), "histc counts")
+        pool(keep2, 2, 2, 0)
+    return "outputs of one rotated set equal PyTorch CPU" + (" (1e-5 relative for the batch-norm statistics)"
+                                                             if name == "bn_upsample" else " bit for bit")
 
 
-def run_search_pair(cfg, name, log2_a, log2_b, sweep, fused_only, iters=2):
-    """sha256d+blake2b (log2 nonces each) or ethash+blake2b."""
+# ------------------------------------------------------------------ searches
+def sha256d_digest(header80: bytes, nonce: int) -> bytes:
+    msg = header80[:76] + int(nonce & 0xFFFFFFFF).to_bytes(4, "little")
+    return hashlib.sha256(hashlib.sha256(msg).digest()).digest()
+
+
+def sia_digest(header80: bytes, nonce: int) -> bytes:
+    msg = header80[:32] + int(nonce & 0xFFFFFFFF).to_bytes(4, "little") + header80[36:]
+    return hashlib.blake2b(msg, digest_size=32).digest()
+
+
+def run_search_pair(cfg, name, log2_a, log2_b, sweep, fused_only, steps=0, warmup=0, iters=2):
+    """sha256d+blake2b or ethash+blake2b over 2^log2_a + 2^log2_b nonces.  With steps > 0 the fused
+    kernel is also run for the contract's timed region: `warmup` untimed launches, then exactly
+    `steps` launches between two synchronisations."""
     import torch
     from hfuse_amd import launcher as H
-    from oracle import oracle as O
     ethash = name == "ethash_blake2b"
     k1 = "ethash_search" if ethash else "sha256d_gpu_hash_shared"
     k2 = "sia_blake2b_gpu_hash"
-    na, nb = 1 << log2_a, 1 << log2_b
-    target32 = (1 << 32) - 1            # 32 leading zero bits
-    hdr_a = O.seeded_bytes(32 if ethash else 80, SEED + 100)
-    hdr_b = O.seeded_bytes(80, SEED + 101)
-    H.sia_blake2b_set_block(hdr_b)
-    keep = []
-    if ethash:
-        n_items = 1 << 25               # 4 GiB of 128-byte items
-        dag = torch.empty(n_items * 32, dtype=torch.int32, device="cuda")
-        H.fill_splitmix64(dag, SEED)
-        torch.cuda.synchronize()
-        eth_target = (1 << 40) - 1      # 24 leading zero bits: ~16 expected hits in 2^28 nonces
-        H.ethash_set_constants(dag, n_items, hdr_a, eth_target)
-        keep.append(dag)
-    else:
-        H.sha256d_set_block(hdr_a, target32)
+    sp = SearchPair(k1, k2, log2_a, log2_b)
+    na, nb = sp.nonces
+    grid = sp.grid          # native Ethash launch of 128-thread blocks over `na` nonces; 0 for the others
+    i = cfg.find_fusion(k1, k2)
 
-    def fresh():
-        ra, rb = H.new_search_results(), H.new_search_results()
-        a1 = H.ethash_args(ra, 0) if ethash else H.sha256d_args(ra, na, 0)
-        a2 = H.blake2b_args(rb, nb, 0, target32)
-        return ra, rb, a1, a2
+    def bound(plan):
+        plan.bind_constants(sp.constants)
+        return plan
 
-    grid = na // 128 if ethash else 0
-    ra, rb, a1, a2 = fresh()
+    ra, rb, a1, a2 = sp.fresh()
     res = {}
-    plans = candidate_plans(cfg, k1, k2, sweep)
+    plans = [(lab, bound(p)) for lab, p in candidate_plans(cfg, k1, k2, sweep)]
     base = plans[0][1]
-    if not fused_only:
-        res["t_a_ms"] = base.time(0, [a1], [a2], 1, iters, grid) / iters
-        res["t_b_ms"] = base.time(1, [a1], [a2], 1, iters, 0) / iters
-        res["t_b2b_ms"] = base.time(2, [a1], [a2], 0, iters, grid) / iters
+
     def grid_of(plan):
         # ethash scans grid * (its share of the fused block) nonces: keep the range at `na`
         if not ethash:
@@ -188,42 +239,91 @@ def run_search_pair(cfg, name, log2_a, log2_b, sweep, fused_only, iters=2):
             best = (t, label, plan)
     _, label, plan = best
     fused_grid = grid_of(plan)
-    res["t_fused_ms"] = plan.time(3, [a1], [a2], 0, iters, fused_grid) / iters
     if not fused_only:
-        res["t_vfuse_ms"] = cfg.plan(cfg.find_fusion(k1, k2), "vfuse").time(3, [a1], [a2], 0, 1, grid)
-        res["t_two_streams_ms"] = base.time(4, [a1], [a2], 0, 1, grid)
-        lbplan = cfg.plan(cfg.find_fusion(k1, k2), "hfuse_lb")
-        res["t_fused_lb_ms"] = lbplan.time(3, [a1], [a2], 0, 1, grid_of(lbplan))
+        vplan, lbplan = bound(cfg.plan(i, "vfuse")), bound(cfg.plan(i, "hfuse_lb"))
+        runs = [("t_a_ms", base, 0, grid), ("t_b_ms", base, 1, 0), ("t_b2b_ms", base, 2, grid),
+                ("t_fused_ms", plan, 3, fused_grid), ("t_two_streams_ms", base, 4, grid),
+                ("t_vfuse_ms", vplan, 3, grid), ("t_fused_lb_ms", lbplan, 3, grid_of(lbplan))]
+    else:
+        runs = [("t_fused_ms", plan, 3, fused_grid)]
+    samples = {k: [] for k, _, _, _ in runs}
+    for _ in range(iters):                       # modes interleaved, one launch per sample
+        for key, p, m, g in runs:
+            samples[key].append(p.time(m, [a1], [a2], 0, 1, g))
+    res.update({k: statistics.median(v) for k, v in samples.items()})
+    if steps > 0:
+        if warmup:
+            plan.time(3, [a1], [a2], 0, warmup, fused_grid)
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        ev_ms = plan.time(3, [a1], [a2], 0, steps, fused_grid)   # HIP events on the launch stream
+        torch.cuda.synchronize()
+        res["wall_ms_per_step"] = (time.perf_counter() - t0) * 1e3 / steps
+        res["event_ms_per_step"] = ev_ms / steps
     res["split"] = label
     part = plan.partition
     res["fused_name"] = part.name.decode()
     res["threads"] = [part.hi[0] - part.lo[0], part.hi[1] - part.lo[1]]
-    # Correctness of what was just timed: one more fused pass into fresh buffers, every hit
-    # re-hashed by the oracle, and the found sets compared with the native kernels' found sets.
-    fa, fb, f1, f2 = fresh()
+    # Correctness of what was just timed: one more fused pass into fresh buffers, the found sets
+    # compared with the native kernels' found sets, SHA-256d and Blake2b hits re-hashed with hashlib.
+    fa, fb, f1, f2 = sp.fresh()
     plan.launch(f1, f2, grid_blocks=fused_grid)
-    na_, nb_, n1, n2 = fresh()
-    H.launch_native(k1, n1, grid, 128)
-    H.launch_native(k2, n2, 0, 128)
+    na_, nb_, n1, n2 = sp.fresh()
+    H.launch_native(k1, n1, grid, 128, constants=sp.constants)
+    H.launch_native(k2, n2, 0, 128, constants=sp.constants)
     torch.cuda.synchronize()
     got_a, got_b = H.read_search_results(fa), H.read_search_results(fb)
     assert got_a == H.read_search_results(na_) and got_b == H.read_search_results(nb_), "fused and native found sets differ"
-    for nonce, digest, mix in got_a[1]:
-        if ethash:
-            assert (mix, digest) == O.ethash_hash(None, SEED, 1 << 25, hdr_a, nonce), "ethash hit differs from the oracle"
-        else:
-            assert digest == O.sha256d_80(hdr_a, nonce), "sha256d hit differs from the oracle"
+    if not ethash:
+        for nonce, digest, _ in got_a[1]:
+            assert digest == sha256d_digest(sp.headers[0], nonce), "sha256d hit differs from hashlib"
     for nonce, digest, _ in got_b[1]:
-        assert digest == O.sia_blake2b_80(hdr_b, nonce & 0xFFFFFFFF), "blake2b hit differs from the oracle"
+        assert digest == sia_digest(sp.headers[1], nonce), "blake2b hit differs from hashlib"
+    # The benchmark's targets leave few or no hits to look at (32 leading zero bits over 2^30 nonces: none
+    # in three runs out of four), so the same fused kernel runs once more over the same ranges with easier
+    # targets (about 16 expected hits each) and those hits are checked the same way.
+    easy = H.Constants()
+    easy_bits = max(4, log2_b - 4)
+    easy_target = (1 << (64 - easy_bits)) - 1
+    if ethash:
+        easy.set_ethash(sp._keep[0], sp.dag_items, sp.headers[0], (1 << (64 - max(4, log2_a - 4))) - 1)
+    else:
+        easy.set_sha256d(sp.headers[0], (1 << (64 - max(4, log2_a - 4))) - 1)
+    easy.set_sia_blake2b(sp.headers[1])
+    ea, eb = H.new_search_results(), H.new_search_results()
+    e1 = H.ethash_args(ea, 0) if ethash else H.sha256d_args(ea, na, 0)
+    e2 = H.blake2b_args(eb, nb, 0, easy_target)
+    eplan = cfg.plan(i)
+    eplan.bind_constants(easy)
+    eplan.launch(e1, e2, grid_blocks=fused_grid)
+    na2, nb2 = H.new_search_results(), H.new_search_results()
+    H.launch_native(k1, H.ethash_args(na2, 0) if ethash else H.sha256d_args(na2, na, 0), grid, 128, constants=easy)
+    H.launch_native(k2, H.blake2b_args(nb2, nb, 0, easy_target), 0, 128, constants=easy)
+    torch.cuda.synchronize()
+    easy_a, easy_b = H.read_search_results(ea), H.read_search_results(eb)
+    assert easy_a == H.read_search_results(na2) and easy_b == H.read_search_results(nb2), \
+        "fused and native found sets differ (easy targets)"
+    if not ethash:
+        for nonce, digest, _ in easy_a[1]:
+            assert digest == sha256d_digest(sp.headers[0], nonce), "sha256d hit differs from hashlib"
+    for nonce, digest, _ in easy_b[1]:
+        assert digest == sia_digest(sp.headers[1], nonce), "blake2b hit differs from hashlib"
     res["hits"] = [got_a[0], got_b[0]]
+    res["hits_easy_targets"] = [easy_a[0], easy_b[0]]
     res["nonces"] = [na, nb]
-    del keep
+    res["check"] = ("fused found sets equal the native kernels' at the benchmark targets and at easier ones; every "
+                    "SHA-256d / Blake2b hit re-hashed with hashlib" + ("; Ethash hits against the CPU restatement in the CPU leg"
+                                                                      if ethash else ""))
+    # kept for the CPU leg, which scans the first part of each range with the CPU restatement
+    res["_found"] = {"a": got_a, "b": got_b, "headers": sp.headers, "dag_items": sp.dag_items}
+    del sp
     return res
 
 
 # ------------------------------------------------------------------ CPU baseline
-def cpu_baseline_tensor(name, budget_s=12.0):
-    """Oracle (C port, OpenMP) and PyTorch CPU ops on the full shape of the pair, repeated within a budget."""
+def cpu_baseline_tensor(name, budget_s=8.0):
+    """PyTorch's CPU operators (the reference CPU path) and the C restatement (OpenMP) on the full shape of
+    the pair, repeated within a budget."""
     import torch
     from oracle import oracle as O
     g = torch.Generator().manual_seed(1)
@@ -257,35 +357,46 @@ def cpu_baseline_tensor(name, budget_s=12.0):
             fn()
             n += 1
         return (time.perf_counter() - t0) / n, n
-    tp, npass = clock(port)
     tr, nref = clock(ref)
-    return dict(port_ms=tp * 1e3, port_gbps=nbytes / tp / 1e9, port_passes=npass,
-                torch_cpu_ms=tr * 1e3, torch_cpu_gbps=nbytes / tr / 1e9, torch_threads=torch.get_num_threads(),
-                threads=O.num_threads())
+    tp, npass = clock(port)
+    return dict(value=nbytes / tr / 1e9, unit="GB/s", kind="reference (PyTorch CPU operators)",
+                cores=torch.get_num_threads(), torch_cpu_ms=tr * 1e3, torch_cpu_passes=nref,
+                port_gbps=nbytes / tp / 1e9, port_ms=tp * 1e3, port_passes=npass, port_threads=O.num_threads())
 
 
-def cpu_baseline_search(name, seconds=6.0):
+def cpu_baseline_search(name, found, log2_a, log2_b):
+    """The CPU restatement of the two searches on a bounded sample of the same ranges: the first 2^k nonces
+    of each, with the benchmark's headers, DAG and targets.  Its found sets must equal what the GPU found
+    in those sub-ranges."""
     from oracle import oracle as O
-    hdr80 = O.seeded_bytes(80, SEED + 101)
+    hdr_a, hdr_b = found["headers"]
     out = {"threads": O.num_threads()}
 
-    def rate(fn, n0):
-        n = n0
-        while True:
-            t0 = time.perf_counter()
-            fn(n)
-            dt = time.perf_counter() - t0
-            if dt > seconds / 3 or n >= 1 << 28:
-                return n / dt / 1e6, n
-            n *= 4
-    out["blake2b_mhs"], out["blake2b_sample"] = rate(lambda n: O.sia_search(hdr80, 0, n, 0), 1 << 18)
+    def scan(fn, n):
+        t0 = time.perf_counter()
+        count, hits = fn(n)
+        dt = time.perf_counter() - t0
+        return n / dt / 1e6, dt, count, [(h.nonce, h.digest_bytes(), h.mix_bytes()) for h in hits]
+
+    def gpu_hits_below(key, n):
+        return [h for h in found[key][1] if (h[0] & 0xFFFFFFFF if key == "b" else h[0]) < n]
+
+    nb = 1 << min(log2_b, 29)             # ~100 MH/s on 16 threads: about 5 s
+    out["blake2b_mhs"], out["blake2b_s"], cnt, hits = scan(lambda n: O.sia_search(hdr_b, 0, n, SearchPair.TARGET32), nb)
+    out["blake2b_sample"] = nb
+    assert hits == gpu_hits_below("b", nb), "Blake2b: CPU and GPU found sets differ in the scanned sub-range"
     if name == "sha256d_blake2b":
-        out["sha256d_mhs"], out["sha256d_sample"] = rate(lambda n: O.sha256d_search(hdr80, 0, n, 0), 1 << 18)
+        na = 1 << min(log2_a, 28)         # ~30 MH/s: about 9 s
+        out["sha256d_mhs"], out["sha256d_s"], cnt, hits = scan(lambda n: O.sha256d_search(hdr_a, 0, n, SearchPair.TARGET32), na)
+        out["sha256d_sample"] = na
+        assert hits == gpu_hits_below("a", na), "SHA-256d: CPU and GPU found sets differ in the scanned sub-range"
     else:
-        hdr32 = O.seeded_bytes(32, SEED + 100)
-        # the same 4 GiB synthetic DAG, evaluated on the fly by the counter generator
-        out["ethash_mhs"], out["ethash_sample"] = rate(
-            lambda n: O.ethash_search(None, SEED, 1 << 25, hdr32, 0, n, 0), 1 << 12)
+        na = 1 << min(log2_a, 26)         # ~6 MH/s with the DAG items evaluated on the fly: about 11 s
+        out["ethash_mhs"], out["ethash_s"], cnt, hits = scan(
+            lambda n: O.ethash_search(None, SEED, found["dag_items"], hdr_a, 0, n, SearchPair.ETHASH_TARGET), na)
+        out["ethash_sample"] = na
+        assert hits == gpu_hits_below("a", na), "Ethash: CPU and GPU found sets (nonce, digest, mix digest) differ in the scanned sub-range"
+        out["ethash_hits_checked"] = len(hits)
     return out
 
 
@@ -314,46 +425,51 @@ def main():
             H.copy_f32(src[i % 4], dst[i % 4])
         torch.cuda.synchronize()
         del src, dst
-    all_names = ["im2col_maxpool", "bn_upsample", "histc_maxpool", "sha256d_blake2b", "ethash_blake2b"]
+    all_names = list(TENSOR_NAMES + SEARCH_NAMES)
     names = all_names if args.pairs == "all" else [n for n in args.pairs.split(",") if n]
     if args.headline not in names:
         names.append(args.headline)
     sweep = args.sweep
     report = {}
 
-    # tensor pairs one at a time (each holds ~1 GiB of rotating buffers)
-    headline = None
-    for name in [n for n in names if n in ("im2col_maxpool", "bn_upsample", "histc_maxpool")]:
+    def timed_region(plan, pair):
+        """The contract's timed region for a tensor headline: exactly K launches between two synchronisations."""
+        pair.time(plan, 3, 0, max(args.warmup, 1))
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        ev_ms = pair.time(plan, 3, 0, args.steps)
+        torch.cuda.synchronize()
+        return (time.perf_counter() - t0) * 1e3 / args.steps, ev_ms / args.steps
+
+    # tensor pairs one at a time (each holds several GiB of rotating buffers)
+    for name in [n for n in names if n in TENSOR_NAMES]:
         pair = build_tensor_pairs([name])[name]
         torch.cuda.synchronize()
-        r = time_tensor_pair(cfg, pair, args.steps, args.warmup, sweep, args.fused_only)
+        r = time_tensor_pair(cfg, pair, args.rotations, sweep, args.fused_only)
         plan = r.pop("plan")
         total = pair.bytes1 + pair.bytes2
         r["bytes"] = [pair.bytes1, pair.bytes2]
         r["fused_gbps"] = total / (r["t_fused_ms"] * 1e-3) / 1e9
         r["roofline_frac"] = r["fused_gbps"] / HBM_PEAK_GBPS
+        r["roofline_bound"] = "hbm"
         if not args.fused_only:
             r["a_gbps"] = pair.bytes1 / (r["t_a_ms"] * 1e-3) / 1e9
             r["b_gbps"] = pair.bytes2 / (r["t_b_ms"] * 1e-3) / 1e9
-            r["speedup_pct"] = (r["t_b2b_ms"] / r["t_fused_ms"] - 1.0) * 100.0
+            judge(r)
         if name == args.headline:
-            # the timed region of the contract: exactly K steps between two synchronisations
-            plan.time(3, pair.args1, pair.args2, args.warmup, 1)
-            torch.cuda.synchronize()
-            t0 = time.perf_counter()
-            ev_ms = plan.time(3, pair.args1, pair.args2, 0, args.steps)
-            torch.cuda.synchronize()
-            wall_ms = (time.perf_counter() - t0) * 1e3
-            headline = dict(r, wall_ms_per_step=wall_ms / args.steps, event_ms_per_step=ev_ms / args.steps,
-                            total_bytes=total, nsets=len(pair.sets))
+            r["wall_ms_per_step"], r["event_ms_per_step"] = timed_region(plan, pair)
+        r["check"] = check_tensor_pair(name, pair, plan)
         report[name] = r
         del pair, plan
         torch.cuda.empty_cache()
 
-    for name in [n for n in names if n in ("sha256d_blake2b", "ethash_blake2b")]:
+    for name in [n for n in names if n in SEARCH_NAMES]:
         la = args.search_log2 or (28 if name == "ethash_blake2b" else 30)
         lb = args.search_log2 + 2 if (args.search_log2 and name == "ethash_blake2b") else (args.search_log2 or 30)
-        r = run_search_pair(cfg, name, la, lb, sweep, args.fused_only)
+        head = name == args.headline
+        r = run_search_pair(cfg, name, la, lb, sweep, args.fused_only, steps=args.steps if head else 0,
+                            warmup=args.warmup if head else 0)
+        r["log2_nonces"] = [la, lb]
         na, nb = r["nonces"]
         tf = r["t_fused_ms"] * 1e-3
         r["fused_mhs"] = [na / tf / 1e6, nb / tf / 1e6]
@@ -370,7 +486,7 @@ def main():
         if not args.fused_only:
             r["a_mhs"] = na / (r["t_a_ms"] * 1e-3) / 1e6
             r["b_mhs"] = nb / (r["t_b_ms"] * 1e-3) / 1e6
-            r["speedup_pct"] = (r["t_b2b_ms"] / r["t_fused_ms"] - 1.0) * 100.0
+            judge(r)
         report[name] = r
         torch.cuda.empty_cache()
 
@@ -381,35 +497,77 @@ def main():
         for _, k1, k2 in cfg.fusions():
             if k1 in tensor_kernels and k2 in tensor_kernels and (k1, k2) not in done:
                 pair = build_pair(f"{k1}+{k2}", k1, k2)
-                r = time_tensor_pair(cfg, pair, args.steps, args.warmup, sweep, False)
+                r = time_tensor_pair(cfg, pair, args.rotations, sweep, False)
                 r.pop("plan")
                 r["fused_gbps"] = (pair.bytes1 + pair.bytes2) / (r["t_fused_ms"] * 1e-3) / 1e9
-                r["speedup_pct"] = (r["t_b2b_ms"] / r["t_fused_ms"] - 1.0) * 100.0
+                judge(r)
                 extra[pair.name] = r
                 del pair
                 torch.cuda.empty_cache()
 
     cpu = None
+    found = {n: report[n].pop("_found") for n in names if n in SEARCH_NAMES}
     if not args.no_cpu:
-        from oracle import oracle as O
         for name in names:
-            if name in ("sha256d_blake2b", "ethash_blake2b"):
-                report[name]["cpu"] = cpu_baseline_search(name)
-            elif name != args.headline:
-                report[name]["cpu"] = cpu_baseline_tensor(name, 8.0)
-        c = cpu_baseline_tensor(args.headline, 16.0)
-        report[args.headline]["cpu"] = c
-        cpu = {"value": c["port_gbps"], "unit": "GB/s", "cores": c["threads"], "kind": "port",
-               "sample": f"{c['port_passes']} full passes of the headline pair's CPU port (oracle, OpenMP) "
-                         f"at {c['port_ms']:.1f} ms each; PyTorch CPU ops on the same tensors: "
-                         f"{c['torch_cpu_gbps']:.2f} GB/s on {c['torch_threads']} threads",
-               "host_cpus": os.cpu_count()}
+            if name in SEARCH_NAMES:
+                report[name]["cpu"] = cpu_baseline_search(name, found[name], *report[name]["log2_nonces"])
+            else:
+                report[name]["cpu"] = cpu_baseline_tensor(name, 12.0 if name == args.headline else 8.0)
+        c = report[args.headline]["cpu"]
+        if args.headline == "ethash_blake2b":
+            cpu = {"value": c["ethash_mhs"], "unit": "MH/s (Ethash)", "cores": c["threads"], "kind": "port",
+                   "sample": f"the first 2^{c['ethash_sample'].bit_length() - 1} of the 2^28 Ethash nonces over the same 4 GiB "
+                             f"synthetic DAG (items evaluated on the fly), {c['ethash_s']:.1f} s, found set equal to the "
+                             f"GPU's there ({c['ethash_hits_checked']} hits); Sia-Blake2b on the first "
+                             f"2^{c['blake2b_sample'].bit_length() - 1} nonces: {c['blake2b_mhs']:.1f} MH/s in {c['blake2b_s']:.1f} s; "
+                             "C restatement of libethash's hashimoto and of Blake2b, OpenMP over all host threads",
+                   "blake2b_mhs": c["blake2b_mhs"], "host_cpus": os.cpu_count()}
+        elif args.headline in TENSOR_NAMES:
+            cpu = {"value": c["value"], "unit": "GB/s", "cores": c["cores"], "kind": "reference",
+                   "sample": f"{c['torch_cpu_passes']} full passes of the pair with PyTorch's CPU operators at "
+                             f"{c['torch_cpu_ms']:.1f} ms each; the C restatement (OpenMP, {c['port_threads']} threads): "
+                             f"{c['port_gbps']:.2f} GB/s", "host_cpus": os.cpu_count()}
+        else:
+            cpu = {"value": c["sha256d_mhs"], "unit": "MH/s (SHA-256d)", "cores": c["threads"], "kind": "port",
+                   "sample": f"the first 2^{c['sha256d_sample'].bit_length() - 1} SHA-256d nonces in {c['sha256d_s']:.1f} s; "
+                             f"Blake2b {c['blake2b_mhs']:.1f} MH/s", "host_cpus": os.cpu_count()}
 
-    h = headline or {}
+    h = report.get(args.headline, {})
     n_fast = sum(1 for r in report.values() if r.get("speedup_pct", -1e9) >= 10.0)
+    if args.headline == "ethash_blake2b":
+        workload = ("configs[4]: ethash_search over a 4 GiB synthetic DAG (2^25 items of 128 B), 2^28 nonces, target 24 leading "
+                    "zero bits + sia_blake2b_gpu_hash, 2^30 nonces, target 32 leading zero bits; one fused launch per step")
+        alg_bytes = h.get("nonces", [0])[0] * ETHASH_BYTES
+        throughput = {"value": h.get("fused_mhs"), "unit": "MH/s [Ethash, Blake2b] in the fused kernel",
+                      "dag_gbps": h.get("dag_gbps")}
+        dtype = "u32/u64"
+    elif args.headline in TENSOR_NAMES:
+        workload = {"im2col_maxpool": "configs[0]: im2col [32,64,56,56] 3x3 + max_pool2d [32,64,112,112] 3x3 s2",
+                    "bn_upsample": "configs[1]: batch_norm_collect_statistics [32,256,28,28] + upsample_nearest2d [32,64,56,56] 2x",
+                    "histc_maxpool": "configs[2]: histc 2^26 -> 1024 bins + max_pool2d [16,128,64,64] 2x2 s2"}[args.headline]
+        alg_bytes = sum(h.get("bytes", [0]))
+        throughput = {"value": h.get("fused_gbps"), "unit": "GB/s (algorithmic bytes of both kernels / fused time)"}
+        dtype = "f32"
+    else:
+        workload = "configs[3]: sha256d 2^30 nonces + sia_blake2b 2^30 nonces, targets 32 leading zero bits"
+        alg_bytes = None
+        throughput = {"value": h.get("fused_mhs"), "unit": "MH/s [SHA-256d, Blake2b] in the fused kernel"}
+        dtype = "u32/u64"
+    ev = h.get("event_ms_per_step")
+    roofline = None
+    if ev and alg_bytes:
+        ach = alg_bytes / (ev * 1e-3) / 1e9
+        roofline = {"bound": "hbm", "achieved": ach, "peak": HBM_PEAK_GBPS, "unit": "GB/s", "frac": ach / HBM_PEAK_GBPS,
+                    "traffic": TRAFFIC_BYTES.get(args.headline), "kernel": h.get("fused_name"),
+                    "algorithmic_bytes_per_launch": alg_bytes, "avg_launch_ms": ev}
+    elif ev and args.headline == "sha256d_blake2b":
+        ops = h["nonces"][0] * OPS_SHA256D + h["nonces"][1] * OPS_BLAKE2B
+        roofline = {"bound": "valu_int32", "achieved": ops / (ev * 1e-3) / 1e12, "peak": VALU_PEAK_GOPS / 1e3, "unit": "Top/s",
+                    "frac": ops / (ev * 1e-3) / 1e9 / VALU_PEAK_GOPS, "traffic": None, "kernel": h.get("fused_name"),
+                    "avg_launch_ms": ev}
     line = {
         "metric": "fused-pair time vs back-to-back launches (speedup %); GB/s or MH/s vs roofline",
-        "value": h.get("speedup_pct"),
+        "value": ((h["t_b2b_ms"] / ev - 1.0) * 100.0) if (ev and "t_b2b_ms" in h) else h.get("speedup_pct"),
         "unit": "%",
         "n_gpus": 1,
         "steps": args.steps,
@@ -418,20 +576,12 @@ def main():
         "higher_is_better": True,
         "scaling": "weak",
         "vs_baseline": None,
-        "dtype": "f32",
-        "data": "synthetic (seeded), inputs resident in HBM, rotating buffer sets",
-        "config": {"workload": "configs[1]: batch_norm_collect_statistics [32,256,28,28] + upsample_nearest2d "
-                               "[32,64,56,56]->[32,64,112,112], one fused launch per step",
-                   "fused_kernel": h.get("fused_name"), "split_threads": h.get("threads"),
-                   "buffer_sets": h.get("nsets")},
-        "throughput": {"value": h.get("fused_gbps"), "unit": "GB/s (algorithmic bytes of both kernels / fused time)"},
+        "dtype": dtype,
+        "data": "synthetic (seeded), inputs resident in HBM" + (", rotating buffer sets" if args.headline in TENSOR_NAMES else ""),
+        "config": {"workload": workload, "fused_kernel": h.get("fused_name"), "split_threads": h.get("threads")},
+        "throughput": throughput,
         "pairs_at_least_10pct_faster": n_fast,
-        "roofline": {"bound": "hbm", "achieved": (h["total_bytes"] / (h["event_ms_per_step"] * 1e-3) / 1e9) if h else None,
-                     "peak": HBM_PEAK_GBPS, "unit": "GB/s",
-                     "frac": (h["total_bytes"] / (h["event_ms_per_step"] * 1e-3) / 1e9 / HBM_PEAK_GBPS) if h else None,
-                     "traffic": HEADLINE_TRAFFIC_BYTES.get(args.headline),
-                     "kernel": h.get("fused_name"), "algorithmic_bytes_per_launch": h.get("total_bytes"),
-                     "avg_launch_ms": h.get("event_ms_per_step")},
+        "roofline": roofline,
         "cpu_baseline": cpu,
         "pairs": report,
     }

@@ -157,7 +157,7 @@ PROTOTYPES = {
     "hf_launch_native": (C.c_int, [C.c_char_p, C.c_void_p, C.c_int, C.c_int, C.c_void_p]),
     "hf_launch_native_with": (C.c_int, [C.c_char_p, C.c_void_p, C.c_void_p, C.c_int, C.c_int, C.c_void_p]),
     "hf_launch_fused": (C.c_int, [C.c_void_p, C.c_void_p, C.c_void_p, C.c_int, C.c_void_p]),
-    "hf_time_pair": (C.c_int, [C.c_void_p, C.c_int, C.POINTER(C.c_void_p), C.POINTER(C.c_void_p), C.c_int,
+    "hf_time_pair": (C.c_int, [C.c_void_p, C.c_int, C.POINTER(C.c_void_p), C.POINTER(C.c_void_p), C.c_int, C.c_int,
                                C.c_int, C.c_int, C.c_int, C.c_void_p, C.POINTER(C.c_float)]),
     "hf_fill_splitmix64": (C.c_int, [C.c_void_p, C.c_uint64, C.c_uint64, C.c_void_p]),
     "hf_copy_f32": (C.c_int, [C.c_void_p, C.c_void_p, C.c_uint64, C.c_void_p]),

@@ -582,7 +582,7 @@ int pairs_only(const FusionRow &f) {
 extern "C" {
 
 HF_API const char *hf_last_error(void) { return g_error.c_str(); }
-HF_API int hf_version(void) { return 100; }
+HF_API int hf_version(void) { return 200; }
 
 HF_API int hf_config_load_text(const char *fusion_yaml, const char *kernels_yaml, hf_config **out) try {
   if (!out) return fail(HF_EINVAL, "null output pointer");
@@ -1130,9 +1130,10 @@ HF_API int hf_launch_fused(const hf_plan *plan, const void *args1, const void *a
 }
 
 HF_API int hf_time_pair(const hf_plan *plan, int mode, const void *const *args1, const void *const *args2, int nsets,
-                        int warmup, int iters, int grid_blocks, void *stream_, float *elapsed_ms) try {
+                        int first_set, int warmup, int iters, int grid_blocks, void *stream_, float *elapsed_ms) try {
   if (!plan || !args1 || !args2 || !elapsed_ms) return fail(HF_EINVAL, "null argument");
-  if (nsets <= 0 || iters <= 0 || warmup < 0 || mode < 0 || mode > 4) return fail(HF_EINVAL, "bad repetition arguments");
+  if (nsets <= 0 || iters <= 0 || warmup < 0 || mode < 0 || mode > 4 || first_set < 0 || first_set >= nsets)
+    return fail(HF_EINVAL, "bad repetition arguments");
   hipStream_t stream = static_cast<hipStream_t>(stream_);
   // mode 4: a second stream (default priority) and a fork / join event pair per repetition
   hipStream_t side = nullptr;
@@ -1162,7 +1163,7 @@ HF_API int hf_time_pair(const hf_plan *plan, int mode, const void *const *args1,
   }
   const unsigned b1 = plan->rows[0].native_block(), b2 = plan->rows[1].native_block();
   auto once = [&](int i) -> int {
-    const int s = i % nsets;
+    const int s = (int)(((long long)first_set + i) % nsets);
     int rc = HF_OK;
     // A kernel whose grid fixes its amount of work (ethash) always gets grid_blocks; the
     // others size their own grid in the back-to-back mode.

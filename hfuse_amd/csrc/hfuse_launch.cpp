@@ -290,7 +290,7 @@ double run_pair(hf_config *cfg, int index, const std::string &preset, int split,
   const char *label[4] = {k1, k2, "back to back", part.name};
   float ms[4];
   for (int mode = 0; mode < 4; mode++) {
-    hf_check(hf_time_pair(plan, mode, a1, a2, 1, 2, iters, mode == 3 ? fused_grid : native_grid, nullptr, &ms[mode]));
+    hf_check(hf_time_pair(plan, mode, a1, a2, 1, 0, 2, iters, mode == 3 ? fused_grid : native_grid, nullptr, &ms[mode]));
     std::printf("%-60s %10.3f us per launch\n", label[mode], 1e3 * ms[mode] / iters);
   }
   const double speedup = (ms[2] / ms[3] - 1.0) * 100.0;

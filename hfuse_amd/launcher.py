@@ -143,16 +143,32 @@ class Plan:
                                       _stream_ptr(stream)))
 
     def time(self, mode: int, args1: Sequence, args2: Sequence, warmup: int, iters: int,
-             grid_blocks: int = 0, stream=None) -> float:
-        """Milliseconds for `iters` repetitions (mode 0/1 native, 2 back-to-back, 3 fused)."""
+             grid_blocks: int = 0, stream=None, rotation: Optional["Rotation"] = None) -> float:
+        """Milliseconds for `iters` repetitions (mode 0/1 native, 2 back-to-back, 3 fused, 4 two streams).
+
+        With a `rotation` the call starts at the buffer set after the last one any earlier call used
+        and moves the cursor on, so short calls keep cycling through all sets."""
         n = len(args1)
         assert n == len(args2) and n > 0
         a1 = (C.c_void_p * n)(*[C.addressof(a) for a in args1])
         a2 = (C.c_void_p * n)(*[C.addressof(a) for a in args2])
         ms = C.c_float()
-        check(L.lib().hf_time_pair(self._h, mode, a1, a2, n, warmup, iters, grid_blocks,
+        first = rotation.take(n, warmup + iters) if rotation is not None else 0
+        check(L.lib().hf_time_pair(self._h, mode, a1, a2, n, first, warmup, iters, grid_blocks,
                                    _stream_ptr(stream), C.byref(ms)))
         return ms.value
+
+
+class Rotation:
+    """Cursor over the buffer sets of a workload, shared by every timing call on them."""
+
+    def __init__(self):
+        self.cursor = 0
+
+    def take(self, nsets: int, launches: int) -> int:
+        first = self.cursor % nsets
+        self.cursor = (first + launches) % nsets
+        return first
 
 
 def launch_native(kernel_name: str, args, grid_blocks: int = 0, block_threads: int = 0, stream=None,

@@ -115,11 +115,13 @@ def tune(cfg: H.Config, fusion_index: int, args1: Sequence, args2: Sequence, *,
          blocks: Optional[Sequence[Tuple[int, int]]] = None, lending: Sequence[bool] = (True, False),
          barrier_modes: Sequence[Optional[int]] = (None,), grids: Sequence[Tuple[int, int]] = ((0, 0),),
          probe_iters: int = 20, final_iters: int = 100, finalists: int = 4, warmup: int = 3,
-         grid_blocks=0, launch_bound: bool = True, verbose: bool = False) -> TuneResult:
+         grid_blocks=0, launch_bound: bool = True, verbose: bool = False,
+         rotation: Optional[H.Rotation] = None) -> TuneResult:
     """Sweep the candidates of one pair on the caller's argument sets and return the fastest.
 
     args1[i] / args2[i] are argument structs of independent buffer sets the timed launches rotate
-    through (hf_time_pair).  Every candidate gets `probe_iters` launches; the `finalists` fastest
+    through (hf_time_pair); every call continues the rotation where the last one stopped, so even a
+    20-launch probe reads buffers that have left the memory-side cache.  Every candidate gets `probe_iters` launches; the `finalists` fastest
     are timed again over `final_iters` launches in three interleaved rounds, together with the
     back-to-back native launches and the untuned table split, and the median decides.  With
     `launch_bound` each finalist also runs in the register-bounded build.
@@ -128,6 +130,8 @@ def tune(cfg: H.Config, fusion_index: int, args1: Sequence, args2: Sequence, *,
     for kernels whose grid fixes their work: Ethash scans grid * its-threads nonces, so a fair
     sweep gives every block shape the grid that covers the same nonce range."""
     grid_of = grid_blocks if callable(grid_blocks) else (lambda t1, t2: grid_blocks)
+    if rotation is None:
+        rotation = H.Rotation()   # one cursor for the whole sweep: short calls keep walking all buffer sets
     file, k1, k2 = cfg.fusion(fusion_index)
     if blocks is None:
         blocks = block_candidates(cfg, fusion_index, step=2 * WAVE)
@@ -139,7 +143,7 @@ def tune(cfg: H.Config, fusion_index: int, args1: Sequence, args2: Sequence, *,
             plan = _make_plan(cfg, fusion_index, c)
         except H.HfuseError:
             continue   # not legal for this pair (BlockDim.Y, barrier mode, block cap)
-        t = plan.time(3, args1, args2, warmup, probe_iters, grid_of(c.threads1, c.threads2)) / probe_iters
+        t = plan.time(3, args1, args2, warmup, probe_iters, grid_of(c.threads1, c.threads2), rotation=rotation) / probe_iters
         probed.append((t, c, plan))
         if verbose:
             print(f"  {c.label():28s} {t * 1e3:9.2f} us", file=sys.stderr, flush=True)
@@ -166,10 +170,11 @@ def tune(cfg: H.Config, fusion_index: int, args1: Sequence, args2: Sequence, *,
     s_b2b, s_table = [], []
     for _ in range(3):
         for i, (_, _, plan) in enumerate(final):
-            samples[i].append(plan.time(3, args1, args2, 2, final_iters, grid_of(final[i][1].threads1, final[i][1].threads2)) / final_iters)
-        s_b2b.append(final[0][2].time(2, args1, args2, 2, final_iters, grid_of(base1, base2)) / final_iters)
+            samples[i].append(plan.time(3, args1, args2, 2, final_iters, grid_of(final[i][1].threads1, final[i][1].threads2),
+                                        rotation=rotation) / final_iters)
+        s_b2b.append(final[0][2].time(2, args1, args2, 2, final_iters, grid_of(base1, base2), rotation=rotation) / final_iters)
         if base_ok:
-            s_table.append(base_cfg_plan.time(3, args1, args2, 2, final_iters, grid_of(base1, base2)) / final_iters)
+            s_table.append(base_cfg_plan.time(3, args1, args2, 2, final_iters, grid_of(base1, base2), rotation=rotation) / final_iters)
     med = sorted(((statistics.median(v), i) for i, v in samples.items()))
     # Timings this close are the same speed: among them prefer the library's defaults
     # (lending on, the pair's own barrier design) so that noise does not write keys.

@@ -40,6 +40,12 @@ class TensorPair:
             read_footprint += s["min_read"]
         self.args1 = [s["a1"] for s in self.sets]
         self.args2 = [s["a2"] for s in self.sets]
+        from .launcher import Rotation
+        self.rotation = Rotation()   # every timing call on this pair continues where the last one stopped
+
+    def time(self, plan, mode, warmup, iters, grid_blocks=0):
+        """Milliseconds of `iters` launches of `plan` in `mode` on this pair's rotating sets."""
+        return plan.time(mode, self.args1, self.args2, warmup, iters, grid_blocks, rotation=self.rotation)
 
 
 def rand(shape, seed, lo=-1.0, hi=1.0, dev="cuda"):

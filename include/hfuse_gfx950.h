@@ -424,11 +424,14 @@ HF_API int hf_launch_fused(const hf_plan *plan, const void *args1, const void *a
  *           (the two-stream launch the reference's traces were taken with)
  * cycling through `nsets` argument sets (args1[i], args2[i]) so repeats do not
  * hit in the last-level cache, and returns the elapsed milliseconds measured
- * with HIP events recorded on `stream` around the timed launches.
+ * with HIP events recorded on `stream` around the timed launches.  Repetition r
+ * (warm-ups included) uses set (first_set + r) % nsets: a caller that times in
+ * several short calls passes the set after the last one used, so that the calls
+ * together keep walking the whole rotation instead of re-reading the first sets.
  */
 HF_API int hf_time_pair(const hf_plan *plan, int mode, const void *const *args1,
-                        const void *const *args2, int nsets, int warmup, int iters,
-                        int grid_blocks, void *stream, float *elapsed_ms);
+                        const void *const *args2, int nsets, int first_set, int warmup,
+                        int iters, int grid_blocks, void *stream, float *elapsed_ms);
 
 /* --------------------------------------------------------- support kernels */
 /* dst[i] = SplitMix64 counter generator word i (seeded synthetic DAG / inputs). */

@@ -242,6 +242,98 @@ def test_every_shipped_search_pair(cuda, cfg):
     assert n == 7
 
 
+def _strict(found_hits, limit, key):
+    """The sub-set of an easy-target found set that also meets the stricter target `limit`."""
+    hits = [h for h in found_hits[1] if key(h[1]) <= limit]
+    return len(hits), hits
+
+
+def test_fused_sha256d_sia_full_benchmark_size(cuda, cfg):
+    """Benchmark configuration 4 at its full size: the fused kernel over 2^30 SHA-256d nonces and 2^30
+    Sia-Blake2b nonces at the 32-leading-zero-bit targets; found sets (most likely empty: P(hit) is 22 % per
+    hash) equal to a full scan by the oracle.  Because an empty set says little about coverage, the same
+    launch is repeated at 26 leading zero bits (about 16 hits per hash expected) against the same scans."""
+    from hfuse_amd.workloads import splitmix64_bytes
+    n = 1 << 30
+    h1, h2 = splitmix64_bytes(80, SEED + 100), splitmix64_bytes(80, SEED + 101)   # the benchmark's headers
+    t32, t26 = (1 << 32) - 1, (1 << 38) - 1
+    easy1 = oracle_hits(O.sha256d_search(h1, 0, n, t26))      # one full scan per hash at the easy target ...
+    easy2 = oracle_hits(O.sia_search(h2, 0, n, t26))
+    assert 1 <= easy1[0] <= 64 and 1 <= easy2[0] <= 64
+    strict1 = _strict(easy1, t32, lambda d: int.from_bytes(d[24:32], "little"))   # ... holds the strict one too
+    strict2 = _strict(easy2, t32, lambda d: int.from_bytes(d[:8], "big"))
+    plan = cfg.plan(cfg.find_fusion("sha256d_gpu_hash_shared", "sia_blake2b_gpu_hash"))
+    for target, want1, want2 in ((t32, strict1, strict2), (t26, easy1, easy2)):
+        c = H.Constants().set_sha256d(h1, target).set_sia_blake2b(h2)
+        plan.bind_constants(c)
+        r1, r2 = H.new_search_results(), H.new_search_results()
+        plan.launch(H.sha256d_args(r1, n, 0), H.blake2b_args(r2, n, 0, target))
+        sync()
+        assert H.read_search_results(r1) == want1, hex(target)
+        assert H.read_search_results(r2) == want2, hex(target)
+
+
+def test_fused_ethash_sia_full_benchmark_size(cuda, cfg):
+    """Benchmark configuration 5 at its full size: Ethash over the 4 GiB synthetic DAG (item byte offsets
+    beyond 2^32), 2^28 nonces at 24 leading zero bits, fused with 2^30 Sia-Blake2b nonces; nonces, final
+    hashes and mix digests equal to a full scan by the oracle over the same DAG (items evaluated on the fly)."""
+    from hfuse_amd.workloads import SearchPair
+    sp = SearchPair("ethash_search", "sia_blake2b_gpu_hash", 28, 30)
+    i = cfg.find_fusion("ethash_search", "sia_blake2b_gpu_hash")
+    plan = cfg.plan(i)
+    plan.bind_constants(sp.constants)
+    r1, r2, a1, a2 = sp.fresh()
+    share = plan.partition.hi[0] - plan.partition.lo[0]
+    plan.launch(a1, a2, grid_blocks=sp.nonces[0] // share)
+    n1 = H.new_search_results()
+    H.launch_native("ethash_search", H.ethash_args(n1, 0), sp.grid, 128, constants=sp.constants)
+    sync()
+    got = H.read_search_results(r1)
+    assert got == H.read_search_results(n1)
+    want = oracle_hits(O.ethash_search(None, SEED, sp.dag_items, sp.headers[0], 0, sp.nonces[0], sp.ETHASH_TARGET))
+    assert 1 <= want[0] <= 64
+    assert got == want
+    # the Blake2b half of the same launch: found set against a full scan (the other full-size test pins
+    # the same 2^30 range at an easier target as well)
+    assert H.read_search_results(r2) == oracle_hits(O.sia_search(sp.headers[1], 0, sp.nonces[1], sp.TARGET32))
+
+
+def test_two_threads_with_their_own_constants(cuda, cfg):
+    """Two host threads search different headers at once, each with its own hf_constants (one bound to a
+    plan, one passed per call) and its own stream: neither sees the other's header."""
+    import threading
+    hdrs = [O.seeded_bytes(80, SEED + 40 + k) for k in range(2)]
+    want = [oracle_hits(O.sha256d_search(h, 0, 1 << 16, EASY12)) for h in hdrs]   # about 16 hits each
+    assert want[0] != want[1] and 0 < want[0][0] < 64 and 0 < want[1][0] < 64
+    i = cfg.find_fusion("sha256d_gpu_hash_shared", "sia_blake2b_gpu_hash")
+    errors = []
+
+    def work(k):
+        try:
+            stream = torch.cuda.Stream()
+            consts = H.Constants().set_sha256d(hdrs[k], EASY12).set_sia_blake2b(hdrs[1 - k])
+            plan = cfg.plan(i)
+            plan.bind_constants(consts)
+            for rep in range(20):
+                r1, r2 = H.new_search_results(), H.new_search_results()
+                with torch.cuda.stream(stream):
+                    if rep % 2:
+                        plan.launch(H.sha256d_args(r1, 1 << 16, 0), H.blake2b_args(r2, 1 << 10, 0, EASY12), stream=stream)
+                    else:
+                        H.launch_native("sha256d_gpu_hash_shared", H.sha256d_args(r1, 1 << 16, 0), stream=stream, constants=consts)
+                stream.synchronize()
+                assert H.read_search_results(r1) == want[k], (k, rep)
+        except Exception as e:   # surfaces in the main thread
+            errors.append(e)
+
+    threads = [threading.Thread(target=work, args=(k,)) for k in range(2)]
+    for t in threads:
+        t.start()
+    for t in threads:
+        t.join()
+    assert not errors, errors
+
+
 def test_zero_nonces_find_nothing(cuda, cfg):
     hdr = O.seeded_bytes(80, SEED + 5)
     H.sha256d_set_block(hdr, EASY12)

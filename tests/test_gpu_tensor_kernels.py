@@ -439,6 +439,50 @@ def test_fused_histc_maxpool(cuda, cfg):
             b.check()
 
 
+def test_fused_histc_maxpool_full_benchmark_size(cuda, cfg):
+    """Benchmark configuration 3 at its full shape through the fused kernel: 2^26 values into 1024 bins
+    next to max_pool2d [16,128,64,64] 2x2 s2; counts, values and argmax against PyTorch CPU and the oracle."""
+    n = 1 << 26
+    g = torch.Generator().manual_seed(11)
+    x = torch.rand(n, generator=g, dtype=torch.float32)
+    i = cfg.find_fusion("kernelHistogram1D", "MaxPoolForward")
+    a, b = Histc(cuda, n, 1024, 0.0, 1.0, x=x), MaxPool(cuda, 16, 128, 64, 64, (2, 2), (2, 2), (0, 0))
+    for plan in (cfg.plan(i), cfg.plan(i, "vfuse")):
+        plan.launch(a.args, b.args)
+        sync()
+        assert a.out.sum().item() == n
+        a.check()
+        b.check()
+
+
+def test_time_pair_continues_the_rotation(cuda, cfg):
+    """hf_time_pair's first_set: repetition r uses set (first_set + r) % nsets, so short calls chained
+    through a Rotation touch every set.  Three sets of a tiny histogram; each launch adds its set's
+    element count to that set's bins, which shows which sets ran."""
+    i = cfg.find_fusion("kernelHistogram1D", "MaxPoolForward")
+    plan = cfg.plan(i)
+    hs = [Histc(cuda, 1000 * (k + 1), 16, 0.0, 1.0, seed=50 + k) for k in range(3)]
+    ps = [MaxPool(cuda, 1, 1, 8, 8, (2, 2), (2, 2), (0, 0), seed=60 + k) for k in range(3)]
+    a1, a2 = [h.args for h in hs], [p.args for p in ps]
+    rot = H.Rotation()
+    plan.time(3, a1, a2, 0, 1, rotation=rot)       # set 0
+    plan.time(3, a1, a2, 1, 1, rotation=rot)       # warm-up on set 1, timed on set 2
+    sync()
+    assert [h.out.sum().item() for h in hs] == [1000.0, 2000.0, 3000.0]
+    plan.time(0, a1, a2, 0, 2, rotation=rot)       # native histogram on sets 0 and 1
+    sync()
+    assert [h.out.sum().item() for h in hs] == [2000.0, 4000.0, 3000.0]
+    assert rot.cursor == 2
+    with pytest.raises(H.HfuseError):
+        check = H.check
+        import ctypes as C
+        n = 3
+        p1 = (C.c_void_p * n)(*[C.addressof(a) for a in a1])
+        p2 = (C.c_void_p * n)(*[C.addressof(a) for a in a2])
+        ms = C.c_float()
+        check(H.L.lib().hf_time_pair(plan._h, 3, p1, p2, n, 3, 0, 1, 0, None, C.byref(ms)))   # first_set out of range
+
+
 @pytest.mark.parametrize("lend", [True, False])
 def test_wave_lending_gives_identical_results(cuda, cfg, lend):
     """Blocks beyond one half's grid: with lending the idle half runs the partner's body,

@@ -129,3 +129,26 @@ def test_splitmix64_known_sequence():
     assert O.splitmix64_at(0, 0) == 0xE220A8397B1DCDAF
     assert O.splitmix64_at(0, 1) == 0x6E789E6AA1B965F4
     assert O.splitmix64_at(0, 2) == 0x06C45D188009454F
+
+
+def test_ethash_search_is_the_brute_force_over_ethash_hash():
+    """orc_ethash_search (compare + collect + sort) against one loop over orc_ethash_hash: same hits, same
+    order, same count, for a window that crosses 2^32 and a target that about one nonce in 16 meets."""
+    seed, n_items = 0x48467573, 1021
+    header = O.seeded_bytes(32, 77)
+    target = (1 << 60) - 1
+    start, count = (1 << 32) - 300, 600
+    want = []
+    for nonce in range(start, start + count):
+        mix, fin = O.ethash_hash(None, seed, n_items, header, nonce)
+        if int.from_bytes(fin[:8], "big") <= target:
+            want.append((nonce, fin, mix))
+    found, hits = O.ethash_search(None, seed, n_items, header, start, count, target)
+    assert 10 < found == len(want)
+    assert [(h.nonce, h.digest_bytes(), h.mix_bytes()) for h in hits] == want
+    # more hits than the caller's capacity: the count is still the total, the kept ones are valid hits
+    found2, hits2 = O.ethash_search(None, seed, n_items, header, start, count, target, 5)
+    assert found2 == found and len(hits2) == 5
+    assert all((h.nonce, h.digest_bytes(), h.mix_bytes()) in want for h in hits2)
+    # an unreachable target finds nothing
+    assert O.ethash_search(None, seed, n_items, header, start, count, 0)[0] == 0
