@@ -43,7 +43,8 @@ VALU_PEAK_GOPS = 256 * 128 * 2.4  # 256 CUs x 128 lanes x 2.4 GHz int32 op/s in 
 # the same counter reads for the plain copy kernel (profiles/tensor_pairs_hbm_traffic.md,
 # profiles/search_pairs_hbm_traffic.md); None where no counter run covers the shape
 TRAFFIC_BYTES = {"bn_upsample": 156.98e6, "im2col_maxpool": 443.28e6, "histc_maxpool": 329.49e6,
-                 "ethash_blake2b": None}
+                 # 2 x 67 042 986 KiB FETCH_SIZE per 2^24 hashes (8 183.9 B per hash), at the benchmark's 2^28
+                 "ethash_blake2b": 2 * 67042985.9 * 1024 * 16}
 
 # textbook primitive-op counts per hash (add / logic / rotate / shift = 1 each)
 OPS_SHA256D = 4336
@@ -96,11 +97,22 @@ def candidate_plans(cfg, k1, k2, sweep):
     return out
 
 
+def blockidx_plan(cfg, i):
+    """The pair as a block-index partition (the fallback design: whole workgroups run one kernel) at the
+    plan's own block shape -- co-scheduling in one launch without a thread partition."""
+    from hfuse_amd import _lib as L
+    plan = cfg.plan(i)
+    plan.set_barrier_mode(L.HF_BARRIER_BLOCKIDX)
+    return plan
+
+
 def judge(res):
     """Adds speedup, the fastest way to run the pair and horizontal-vs-vertical to a per-pair result."""
     res["speedup_pct"] = (res["t_b2b_ms"] / res["t_fused_ms"] - 1.0) * 100.0
     ways = {"back_to_back": res["t_b2b_ms"], "two_streams": res["t_two_streams_ms"], "vfuse": res["t_vfuse_ms"],
             "hfuse": res["t_fused_ms"], "hfuse_lb": res["t_fused_lb_ms"]}
+    if "t_blockidx_ms" in res:
+        ways["blockidx"] = res["t_blockidx_ms"]
     res["best_mode"] = min(ways, key=ways.get)
     res["hfuse_vs_vfuse_pct"] = (res["t_vfuse_ms"] / res["t_fused_ms"] - 1.0) * 100.0
     res["hfuse_vs_two_streams_pct"] = (res["t_two_streams_ms"] / res["t_fused_ms"] - 1.0) * 100.0
@@ -131,7 +143,8 @@ def time_tensor_pair(cfg, pair, rotations, sweep, fused_only, rounds=5):
         runs = [("t_a_ms", plan, 0), ("t_b_ms", plan, 1), ("t_b2b_ms", plan, 2), ("t_fused_ms", plan, 3),
                 ("t_two_streams_ms", plan, 4),                     # the launch pattern of the reference's own traces
                 ("t_vfuse_ms", cfg.plan(i, "vfuse"), 3),           # the reference's vertical baseline
-                ("t_fused_lb_ms", cfg.plan(i, "hfuse_lb"), 3)]     # the same block shape, register-bounded build
+                ("t_fused_lb_ms", cfg.plan(i, "hfuse_lb"), 3),     # the same block shape, register-bounded build
+                ("t_blockidx_ms", blockidx_plan(cfg, i), 3)]       # each workgroup runs one of the two kernels
     for _, p, m in runs:                                            # one untimed rotation per mode
         pair.time(p, m, 0, nsets)
     samples = {k: [] for k, _, _ in runs}
@@ -140,6 +153,8 @@ def time_tensor_pair(cfg, pair, rotations, sweep, fused_only, rounds=5):
             samples[key].append(pair.time(p, m, 2, per) / per)
     res = {k: statistics.median(v) for k, v in samples.items()}
     res["launches_per_sample"], res["rounds"], res["buffer_sets"] = per, rounds, nsets
+    if not fused_only:
+        res["lb_waves_per_simd"] = runs[6][1].launch_waves[1]
     res["split"] = label
     part = plan.partition
     res["fused_name"] = part.name.decode()
@@ -251,6 +266,8 @@ def run_search_pair(cfg, name, log2_a, log2_b, sweep, fused_only, steps=0, warmu
         for key, p, m, g in runs:
             samples[key].append(p.time(m, [a1], [a2], 0, 1, g))
     res.update({k: statistics.median(v) for k, v in samples.items()})
+    if not fused_only:
+        res["lb_waves_per_simd"] = lbplan.launch_waves[1]
     if steps > 0:
         if warmup:
             plan.time(3, [a1], [a2], 0, warmup, fused_grid)

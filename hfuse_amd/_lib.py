@@ -139,6 +139,8 @@ PROTOTYPES = {
     "hf_plan_set_grids": (C.c_int, [C.c_void_p, C.c_int, C.c_int]),
     "hf_plan_set_lending": (C.c_int, [C.c_void_p, C.c_int]),
     "hf_plan_set_launch_bound": (C.c_int, [C.c_void_p, C.c_int]),
+    "hf_plan_set_launch_waves": (C.c_int, [C.c_void_p, C.c_int]),
+    "hf_plan_launch_waves": (C.c_int, [C.c_void_p, C.POINTER(C.c_int), C.POINTER(C.c_int)]),
     "hf_plan_set_block": (C.c_int, [C.c_void_p, C.c_int, C.c_int]),
     "hf_plan_partition": (C.c_int, [C.c_void_p, C.POINTER(Partition)]),
     "hf_plan_num_splits": (C.c_int, [C.c_void_p, C.c_int]),

@@ -567,9 +567,30 @@ struct hf_plan {
   unsigned grid_override[2] = {0, 0};  // hf_plan_set_grids
   bool lending = true;                 // hf_plan_set_lending
   int bounded = -1;                    // hf_plan_set_launch_bound: 0 / 1, -1 = by the preset
+  int bound_waves = 0;                 // hf_plan_set_launch_waves: waves per SIMD of the bounded build, 0 = by the formula
 };
 
 namespace {
+// Waves per SIMD the occupancy formula of the reference's printer asks for with this part's constants:
+// B = min_k(regfile / Reg_k / threads_k) blocks per CU, capped by the resident threads
+// (lib/KernelFuser/KernelPrinter.cpp:44-66), times the block's waves, spread over four SIMDs.
+int formula_waves(const hf_plan *plan) {
+  const unsigned long long w = (unsigned long long)plan->part.bound_blocks * plan->part.launch_threads / (4ull * kWave);
+  return (int)std::min<unsigned long long>(std::max<unsigned long long>(w, 1), (unsigned long long)kBoundedWaves);
+}
+
+// The build a launch of this plan runs: 0 = plain, otherwise the wave bound of a register-bounded build.
+// The launch-bound presets ask for a bounded build when the formula wants more waves per SIMD than the
+// plain build's launch bound of 1024 threads already guarantees (four).
+int plan_build_waves(const hf_plan *plan) {
+  if (!plan->preset->base_line && plan->barrier_mode == HF_BARRIER_BLOCKIDX) return 0;  // no bounded build
+  const int formula = formula_waves(plan);
+  const bool want = plan->bounded >= 0 ? plan->bounded != 0 : plan->preset->launch_bound && formula > 4;
+  if (!want) return 0;
+  const int built = built_bound_waves(plan->ids[0], plan->ids[1], plan->bound_waves ? plan->bound_waves : formula);
+  return plan->preset->base_line ? kBoundedWaves : built;   // the vertical baseline has the 8-wave build only
+}
+
 // The reference's Context partitions a block among any number of kernels (include/KernelFusion.h:45-80;
 // configs/crypt_four.yaml fuses three); fused kernels are built for pairs here.
 int pairs_only(const FusionRow &f) {
@@ -825,6 +846,25 @@ HF_API int hf_plan_set_launch_bound(hf_plan *plan, int on) try {
   return trap_exception();
 }
 
+HF_API int hf_plan_set_launch_waves(hf_plan *plan, int waves) try {
+  if (!plan) return fail(HF_EINVAL, "null plan");
+  if (waves < 0 || waves > kBoundedWaves) return fail(HF_EINVAL, "waves per SIMD must be 0 (by the formula) or 1..8");
+  plan->bound_waves = waves;
+  if (waves > 0) plan->bounded = 1;
+  return HF_OK;
+} catch (...) {
+  return trap_exception();
+}
+
+HF_API int hf_plan_launch_waves(const hf_plan *plan, int *formula, int *built) try {
+  if (!plan) return fail(HF_EINVAL, "null plan");
+  if (formula) *formula = formula_waves(plan);
+  if (built) *built = plan_build_waves(plan);
+  return HF_OK;
+} catch (...) {
+  return trap_exception();
+}
+
 HF_API void hf_plan_free(hf_plan *plan) { delete plan; }
 
 HF_API int hf_plan_partition(const hf_plan *plan, hf_partition *out) try {
@@ -1043,12 +1083,7 @@ int do_launch_fused(const hf_plan *plan, const Prepared &p1, const Prepared &p2,
   if ((unsigned long long)std::max(exact, std::max(plan->grid_override[0], plan->grid_override[1])) * (g.d1 + g.d2) >
       0xFFFFFFFFull)
     return fail(HF_EINVAL, "grid_blocks * block threads must fit 32 bits (the bodies index work items with 32-bit counters)");
-  // The launch-bound presets run the register-bounded build whenever their block count asks for
-  // more waves per SIMD than the plain build's launch bound already guarantees.
-  const bool bounded = plan->bounded >= 0
-                           ? plan->bounded != 0
-                           : plan->preset->launch_bound &&
-                                 (unsigned long long)plan->part.launch_blocks * plan->part.launch_threads > 4ull * 256ull;
+  const int waves = plan_build_waves(plan);  // 0: the plain build
   // every thread of the launch may run either body (lending), so each 32-bit counter is checked against all of them
   auto counters_fit = [&](unsigned grid, unsigned block) {
     const unsigned long long threads = (unsigned long long)grid * block;
@@ -1063,8 +1098,8 @@ int do_launch_fused(const hf_plan *plan, const Prepared &p1, const Prepared &p2,
     const size_t lds = 4 * kBarrierWords + g.lds1 + g.lds2;
     const unsigned grid = std::max(g.grid1, g.grid2);
     if (!counters_fit(grid, block)) return fail(HF_EINVAL, kCounterMsg);
-    e = crypto ? launch_fused_crypto(plan->ids[0], plan->ids[1], MODE_VERTICAL, bounded, p1.blob, p2.blob, g, grid, lds, stream)
-               : launch_fused_dl(plan->ids[0], plan->ids[1], MODE_VERTICAL, bounded, p1.blob, p2.blob, g, grid, lds, stream);
+    e = crypto ? launch_fused_crypto(plan->ids[0], plan->ids[1], MODE_VERTICAL, waves, p1.blob, p2.blob, g, grid, lds, stream)
+               : launch_fused_dl(plan->ids[0], plan->ids[1], MODE_VERTICAL, waves, p1.blob, p2.blob, g, grid, lds, stream);
   } else if (plan->barrier_mode == HF_BARRIER_BLOCKIDX) {
     // Each kernel gets its own workgroups inside one launch.
     const unsigned block = std::max(g.d1, g.d2);
@@ -1077,8 +1112,8 @@ int do_launch_fused(const hf_plan *plan, const Prepared &p1, const Prepared &p2,
     const size_t lds = std::max(g.lds1, g.lds2);
     if ((unsigned long long)g.grid1 + g.grid2 > 0xFFFFFFFFull || !counters_fit(g.grid1 + g.grid2, block))
       return fail(HF_EINVAL, kCounterMsg);
-    e = crypto ? launch_fused_crypto(plan->ids[0], plan->ids[1], MODE_BLOCKIDX, false, p1.blob, p2.blob, g, g.grid1 + g.grid2, lds, stream)
-               : launch_fused_dl(plan->ids[0], plan->ids[1], MODE_BLOCKIDX, false, p1.blob, p2.blob, g, g.grid1 + g.grid2, lds, stream);
+    e = crypto ? launch_fused_crypto(plan->ids[0], plan->ids[1], MODE_BLOCKIDX, 0, p1.blob, p2.blob, g, g.grid1 + g.grid2, lds, stream)
+               : launch_fused_dl(plan->ids[0], plan->ids[1], MODE_BLOCKIDX, 0, p1.blob, p2.blob, g, g.grid1 + g.grid2, lds, stream);
   } else {
     // One grid for both halves.  When the caller names it, both halves stride over all of it
     // (a kernel whose grid fixes its work, ethash, always does); otherwise each half strides
@@ -1106,8 +1141,8 @@ int do_launch_fused(const hf_plan *plan, const Prepared &p1, const Prepared &p2,
     if (!counters_fit(grid, block)) return fail(HF_EINVAL, kCounterMsg);
     const size_t lds = 4 * kBarrierWords + g.lds1 + g.lds2;
     const FuseMode mode = plan->barrier_mode == HF_BARRIER_MATCHED ? MODE_MATCHED : MODE_HFUSE;
-    e = crypto ? launch_fused_crypto(plan->ids[0], plan->ids[1], mode, bounded, p1.blob, p2.blob, g, grid, lds, stream)
-               : launch_fused_dl(plan->ids[0], plan->ids[1], mode, bounded, p1.blob, p2.blob, g, grid, lds, stream);
+    e = crypto ? launch_fused_crypto(plan->ids[0], plan->ids[1], mode, waves, p1.blob, p2.blob, g, grid, lds, stream)
+               : launch_fused_dl(plan->ids[0], plan->ids[1], mode, waves, p1.blob, p2.blob, g, grid, lds, stream);
   }
   if (e == hipErrorNotSupported) return fail(HF_EUNSUPPORTED, "this pair / barrier mode is not built");
   if (e != hipSuccess) return hip_fail(e, "fused launch");

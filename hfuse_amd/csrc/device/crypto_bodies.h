@@ -93,6 +93,7 @@ __device__ __forceinline__ void sha256_compress(u32 st[8], u32 w[16]) {
 }
 
 struct Sha256dBody {
+  static constexpr KernelId kId = K_SHA256D;
   using Args = Sha256dDevArgs;
   static constexpr bool kBarriers = false;
   static constexpr bool kFlat = true;
@@ -220,6 +221,7 @@ __device__ __forceinline__ void blake2b_record(const Blake2bDevArgs &a, u32 nonc
 // word 4 (byte 32); ccminer's layout in the high half of word 9 (byte 76).
 template <int NONCE_WORD, bool NONCE_HIGH>
 struct Blake2bBody {
+  static constexpr KernelId kId = NONCE_HIGH ? K_BLAKE2B : K_SIA_BLAKE2B;
   using Args = Blake2bDevArgs;
   static constexpr bool kBarriers = false;
   static constexpr bool kFlat = true;
@@ -314,6 +316,7 @@ __device__ __forceinline__ u32 fnv_reduce(u32x4 v) { return fnv(fnv(fnv(v.x, v.y
 // a group reads one whole item per access.  Four hashes of the group are in
 // flight together to keep four independent gathers outstanding per lane.
 struct EthashBody {
+  static constexpr KernelId kId = K_ETHASH;
   using Args = EthashDevArgs;
   static constexpr bool kBarriers = false;
   static constexpr bool kFlat = false;  // one nonce per thread of the launch grid

@@ -62,6 +62,7 @@ __device__ __forceinline__ void st4(float *p, f32x4 v) {
 // rows channel_in*kh*kw + i*kw + j of the column matrix, zero outside the image.
 // ----------------------------------------------------------------------------
 struct Im2colBody {
+  static constexpr KernelId kId = K_IM2COL;
   using Args = hf_im2col_args;
   static constexpr bool kBarriers = false;
   static constexpr bool kFlat = true;  // walks one flat index range: may borrow a partner's idle waves
@@ -165,6 +166,7 @@ struct Im2colBody {
 // on `v > max || isnan(v)`, so ties keep the first index; the mask is h*W+w.
 // ----------------------------------------------------------------------------
 struct MaxPoolBody {
+  static constexpr KernelId kId = K_MAXPOOL;
   using Args = hf_maxpool_args;
   static constexpr bool kBarriers = false;
   static constexpr bool kFlat = true;
@@ -312,6 +314,7 @@ struct MaxPoolBody {
 // upsample_nearest2d_out_frame<float>: src = min((int)floorf(dst * scale), in - 1)
 // ----------------------------------------------------------------------------
 struct UpsampleNearestBody {
+  static constexpr KernelId kId = K_UPSAMPLE_NEAREST;
   using Args = hf_upsample_nearest_args;
   static constexpr bool kBarriers = false;
   static constexpr bool kFlat = true;
@@ -399,6 +402,7 @@ __device__ __forceinline__ float rn_sub(float x, float y) {
 }
 
 struct UpsampleBilinearBody {
+  static constexpr KernelId kId = K_UPSAMPLE_BILINEAR;
   using Args = hf_upsample_bilinear_args;
   static constexpr bool kBarriers = false;
   static constexpr bool kFlat = true;
@@ -606,6 +610,7 @@ __device__ __forceinline__ Welford wave_merge(Welford w) {
 }
 
 struct BnStatsBody {
+  static constexpr KernelId kId = K_BNSTATS;
   using Args = hf_bn_stats_args;
   static constexpr bool kBarriers = true;
   static constexpr bool kFlat = false;  // one plane per block: the block index is part of the work mapping
@@ -686,6 +691,7 @@ struct BnStatsBody {
 // flush to the fp32 counts with global atomics.
 // ----------------------------------------------------------------------------
 struct HistcBody {
+  static constexpr KernelId kId = K_HISTC;
   using Args = hf_histc_args;
   static constexpr bool kBarriers = true;
   static constexpr bool kFlat = false;  // block-private LDS bins
@@ -763,9 +769,22 @@ struct HistcBody {
       if (sb.bid == 0 && (int64_t)sb.tid < head) count<POW2, GLOBAL>(bins, b[sb.tid], lo, hi, fn, range, inv_range, inv_lo, inv_hi, nbins);
       b += head;
       const int64_t rest = total - head;
+#ifndef HF_HIST_CONTIG
+#define HF_HIST_CONTIG 0
+#endif
+#if HF_HIST_CONTIG
+      // every workgroup walks one contiguous run of the input (a whole number of block-wide rows)
+      const int64_t nall = rest >> 2;
+      const int64_t rows = (nall + sb.nthreads - 1) / sb.nthreads;
+      const int64_t per = (rows + sb.nblocks - 1) / sb.nblocks * sb.nthreads;
+      const int64_t n4 = min(nall, (int64_t)(sb.bid + 1) * per);
+      const int64_t stride = (int64_t)sb.nthreads;
+      int64_t i = (int64_t)sb.bid * per + sb.tid;
+#else
       const int64_t n4 = rest >> 2;
       const int64_t stride = (int64_t)sb.gstride();
       int64_t i = (int64_t)sb.gtid();
+#endif
       // Several 16-byte loads in flight per lane before the dependent LDS atomics: eight with up to
       // eight wavefronts, four with more (about 48-64 KB in flight per CU either way; beyond that the
       // memory system gets slower, and more wavefronts with shorter batches overlap their arithmetic better).
@@ -783,7 +802,7 @@ struct HistcBody {
       else batches(std::integral_constant<int, 8>());
       for (; i < n4; i += stride) count4(ld4_stream(b + i * 4));
       if (sb.bid == 0)
-        for (int64_t k = (n4 << 2) + sb.tid; k < rest; k += sb.nthreads)
+        for (int64_t k = ((rest >> 2) << 2) + sb.tid; k < rest; k += sb.nthreads)
           count<POW2, GLOBAL>(bins, b[k], lo, hi, fn, range, inv_range, inv_lo, inv_hi, nbins);
     } else {
       const int64_t stride = (int64_t)sb.gstride();

@@ -29,6 +29,37 @@ typedef unsigned int u32x2 __attribute__((ext_vector_type(2)));
 
 enum { BAR_WORKGROUP = 0, BAR_SUBSET = 1 };
 
+enum KernelId {
+  K_IM2COL = 0,
+  K_MAXPOOL,
+  K_BNSTATS,
+  K_UPSAMPLE_NEAREST,
+  K_HISTC,
+  K_ETHASH,
+  K_SHA256D,
+  K_SIA_BLAKE2B,
+  K_BLAKE2B,
+  K_UPSAMPLE_BILINEAR,
+  K_COUNT
+};
+
+// Register-bounded builds.  Every pair has one for kBoundedWaves waves per SIMD; the benchmarked
+// pairs whose occupancy formula (min over the kernels of regfile / Reg / threads, capped by the
+// resident threads: lib/KernelFuser/KernelPrinter.cpp:44-66, with this part's 128 K registers and
+// 2048 threads per CU) asks for fewer waves have a second build at exactly that bound.
+constexpr int kBoundedWaves = 8;
+constexpr int pair_extra_waves(KernelId k1, KernelId k2) {
+  return (k1 == K_IM2COL && k2 == K_MAXPOOL) ? 5      // 2 blocks of 256 + 448 threads
+         : (k1 == K_HISTC && k2 == K_MAXPOOL) ? 7     // 2 blocks of 768 + 128
+         : (k1 == K_ETHASH && k2 == K_SIA_BLAKE2B) ? 6  // 8 blocks of 128 + 64
+                                                   : 0;
+}
+// The bound of the build that runs when `waves` waves per SIMD are asked for (0: the plain build).
+constexpr int built_bound_waves(KernelId k1, KernelId k2, int waves) {
+  return waves <= 0 ? 0 : (pair_extra_waves(k1, k2) != 0 && waves <= pair_extra_waves(k1, k2)) ? pair_extra_waves(k1, k2) : kBoundedWaves;
+}
+
+
 template <int BAR>
 struct SubBlock {
   unsigned tid;       // thread index inside this half
@@ -80,12 +111,30 @@ struct FuseGeom {
 
 constexpr unsigned kBarrierWords = 4;  // 16 bytes reserved at the base of LDS for arrival counters
 
+// Workgroups are dealt to the eight XCDs round-robin by their index.  This renumbering gives the
+// workgroups of one XCD consecutive virtual indices: XCD x owns the x-th contiguous eighth of the
+// index range (the first grid % 8 XCDs hold one workgroup more).
+constexpr unsigned kXcds = 8;
+__device__ __forceinline__ unsigned xcd_contiguous(unsigned bid, unsigned grid) {
+  const unsigned xcd = bid % kXcds, slot = bid / kXcds;
+  const unsigned q = grid / kXcds, r = grid % kXcds;
+  return xcd * q + (xcd < r ? xcd : r) + slot;
+}
+
 // Native launch: the body owns the whole workgroup.
 template <class K, int T>
 __global__ __launch_bounds__(T) void native_kernel(typename K::Args a, unsigned hint) {
   extern __shared__ __align__(16) unsigned char smem[];
-  SubBlock<BAR_WORKGROUP> sb{threadIdx.x, blockDim.x, blockIdx.x, gridDim.x, nullptr, 0,
-                             blockIdx.x * blockDim.x, gridDim.x * blockDim.x};
+#ifndef HF_XCD_SWIZZLE
+#define HF_XCD_SWIZZLE 0
+#endif
+#if HF_XCD_SWIZZLE
+  const unsigned bid = xcd_contiguous(blockIdx.x, gridDim.x);
+#else
+  const unsigned bid = blockIdx.x;
+#endif
+  SubBlock<BAR_WORKGROUP> sb{threadIdx.x, blockDim.x, bid, gridDim.x, nullptr, 0,
+                             bid * blockDim.x, gridDim.x * blockDim.x};
   K::run(a, sb, smem, hint);
 }
 
@@ -158,11 +207,9 @@ __global__ __launch_bounds__(T) void fused_kernel(typename K1::Args a1, typename
 // thread limit (lib/KernelFuser/KernelPrinter.cpp:44-66), i.e. it makes the compiler keep the
 // fused kernel's registers low enough for the occupancy the natives had.  The gfx950 form of
 // that request is a waves-per-SIMD bound: this build of each fused kernel is compiled for
-// kBoundedWaves waves per SIMD (at most 512 / 8 = 64 vector registers), spilling if it must.
-constexpr int kBoundedWaves = 8;
-
-template <class K1, class K2, int T, bool MATCHED>
-__global__ __launch_bounds__(T) __attribute__((amdgpu_waves_per_eu(kBoundedWaves, kBoundedWaves)))
+// W waves per SIMD (at most 512 / W vector registers: 64 for the default of 8), spilling if it must.
+template <class K1, class K2, int T, bool MATCHED, int W = kBoundedWaves>
+__global__ __launch_bounds__(T) __attribute__((amdgpu_waves_per_eu(W, W)))
 void fused_kernel_lb(typename K1::Args a1, typename K2::Args a2, FuseGeom g) {
   fused_block<K1, K2, MATCHED>(a1, a2, g);
 }
@@ -220,8 +267,8 @@ __global__ __launch_bounds__(T) void vertical_kernel(typename K1::Args a1, typen
   vertical_block<K1, K2>(a1, a2, g);
 }
 
-template <class K1, class K2, int T>
-__global__ __launch_bounds__(T) __attribute__((amdgpu_waves_per_eu(kBoundedWaves, kBoundedWaves)))
+template <class K1, class K2, int T, int W = kBoundedWaves>
+__global__ __launch_bounds__(T) __attribute__((amdgpu_waves_per_eu(W, W)))
 void vertical_kernel_lb(typename K1::Args a1, typename K2::Args a2, FuseGeom g) {
   vertical_block<K1, K2>(a1, a2, g);
 }

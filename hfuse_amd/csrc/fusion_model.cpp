@@ -304,6 +304,7 @@ int make_partition(const KernelRow &k1, const KernelRow &k2, const Preset &prese
   max_block = std::min(max_block, kMaxResidentThreads / sum);
   out.launch_threads = preset.base_line ? max_thread : sum;
   out.launch_blocks = preset.launch_bound ? max_block : 0;
+  out.bound_blocks = max_block;
   out.name = k1.name + "_" + k2.name + "_fused_kernel_" + variant;  // KernelPrinter.cpp:67-70
   return HF_OK;
 }

@@ -54,6 +54,7 @@ struct Partition {
   uint32_t lo[2], hi[2];
   Dim3 block_dim[2];
   uint32_t launch_threads = 0, launch_blocks = 0;
+  uint32_t bound_blocks = 0;  // the printer's min-blocks value whatever the preset (launch_blocks is 0 without LaunchBound)
   std::string name;  // <K1>_<K2>_fused_kernel_<preset>_idx_<n>
 };
 

@@ -19,13 +19,23 @@ hipError_t native(const void *args, unsigned hint, unsigned grid, unsigned block
 }
 
 template <class K1, class K2>
-hipError_t pair(FuseMode mode, bool bounded, const void *a1, const void *a2, const FuseGeom &g, unsigned grid, size_t lds,
+hipError_t pair(FuseMode mode, int waves, const void *a1, const void *a2, const FuseGeom &g, unsigned grid, size_t lds,
                 hipStream_t s) {
   const auto &x1 = *static_cast<const typename K1::Args *>(a1);
   const auto &x2 = *static_cast<const typename K2::Args *>(a2);
   if (g.d1 + g.d2 > (unsigned)kCryptoBlock) return hipErrorNotSupported;
+  constexpr int kExtra = pair_extra_waves(K1::kId, K2::kId);   // a second bounded build of this pair, or 0
+  const int build = built_bound_waves(K1::kId, K2::kId, waves);
+  const bool bounded = build != 0;
   switch (mode) {
     case MODE_HFUSE:
+      if constexpr (kExtra != 0) {
+        if (build == kExtra) {
+          hipLaunchKernelGGL((fused_kernel_lb<K1, K2, kCryptoBlock, false, kExtra>), dim3(grid), dim3(g.d1 + g.d2), lds, s,
+                             x1, x2, g);
+          break;
+        }
+      }
       if (bounded)
         hipLaunchKernelGGL((fused_kernel_lb<K1, K2, kCryptoBlock, false>), dim3(grid), dim3(g.d1 + g.d2), lds, s, x1,
                            x2, g);
@@ -65,10 +75,10 @@ hipError_t launch_native_crypto(KernelId k, const void *args, unsigned hint, uns
 }
 
 #define HF_PAIR(A, KA, B, KB)                                                     \
-  if (k1 == A && k2 == B) return pair<KA, KB>(mode, bounded, a1, a2, g, grid, lds, s);     \
-  if (k1 == B && k2 == A) return pair<KB, KA>(mode, bounded, a1, a2, g, grid, lds, s);
+  if (k1 == A && k2 == B) return pair<KA, KB>(mode, waves, a1, a2, g, grid, lds, s);     \
+  if (k1 == B && k2 == A) return pair<KB, KA>(mode, waves, a1, a2, g, grid, lds, s);
 
-hipError_t launch_fused_crypto(KernelId k1, KernelId k2, FuseMode mode, bool bounded, const void *a1, const void *a2,
+hipError_t launch_fused_crypto(KernelId k1, KernelId k2, FuseMode mode, int waves, const void *a1, const void *a2,
                                const FuseGeom &g, unsigned grid, size_t lds, hipStream_t s) {
   HF_PAIR(K_ETHASH, EthashBody, K_BLAKE2B, CcminerBlake2bBody)
   HF_PAIR(K_SHA256D, Sha256dBody, K_ETHASH, EthashBody)

@@ -40,23 +40,23 @@ hipError_t launch_native_dl(KernelId k, const void *args, unsigned hint, unsigne
   }
 }
 
-hipError_t launch_fused_dl_a(KernelId k1, KernelId k2, FuseMode mode, bool bounded, const void *a1, const void *a2,
+hipError_t launch_fused_dl_a(KernelId k1, KernelId k2, FuseMode mode, int waves, const void *a1, const void *a2,
                              const FuseGeom &g, unsigned grid, size_t lds, hipStream_t s) {
   switch (k1) {
-    case K_IM2COL: return dl_second<Im2colBody>(k2, mode, bounded, a1, a2, g, grid, lds, s);
-    case K_MAXPOOL: return dl_second<MaxPoolBody>(k2, mode, bounded, a1, a2, g, grid, lds, s);
+    case K_IM2COL: return dl_second<Im2colBody>(k2, mode, waves, a1, a2, g, grid, lds, s);
+    case K_MAXPOOL: return dl_second<MaxPoolBody>(k2, mode, waves, a1, a2, g, grid, lds, s);
     default: return hipErrorNotSupported;
   }
 }
 
-hipError_t launch_fused_dl(KernelId k1, KernelId k2, FuseMode mode, bool bounded, const void *a1, const void *a2, const FuseGeom &g,
+hipError_t launch_fused_dl(KernelId k1, KernelId k2, FuseMode mode, int waves, const void *a1, const void *a2, const FuseGeom &g,
                            unsigned grid, size_t lds, hipStream_t s) {
   switch (k1) {
     case K_IM2COL:
-    case K_MAXPOOL: return launch_fused_dl_a(k1, k2, mode, bounded, a1, a2, g, grid, lds, s);
+    case K_MAXPOOL: return launch_fused_dl_a(k1, k2, mode, waves, a1, a2, g, grid, lds, s);
     case K_BNSTATS:
-    case K_UPSAMPLE_NEAREST: return launch_fused_dl_b(k1, k2, mode, bounded, a1, a2, g, grid, lds, s);
-    default: return launch_fused_dl_c(k1, k2, mode, bounded, a1, a2, g, grid, lds, s);
+    case K_UPSAMPLE_NEAREST: return launch_fused_dl_b(k1, k2, mode, waves, a1, a2, g, grid, lds, s);
+    default: return launch_fused_dl_c(k1, k2, mode, waves, a1, a2, g, grid, lds, s);
   }
 }
 

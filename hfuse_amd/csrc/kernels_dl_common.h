@@ -18,21 +18,29 @@ hipError_t dl_native(const void *args, unsigned hint, unsigned grid, unsigned bl
 }
 
 template <class K1, class K2>
-hipError_t dl_pair(FuseMode mode, bool bounded, const void *a1, const void *a2, const FuseGeom &g, unsigned grid, size_t lds,
+hipError_t dl_pair(FuseMode mode, int waves, const void *a1, const void *a2, const FuseGeom &g, unsigned grid, size_t lds,
                    hipStream_t s) {
   const auto &x1 = *static_cast<const typename K1::Args *>(a1);
   const auto &x2 = *static_cast<const typename K2::Args *>(a2);
   const unsigned wide = g.d1 > g.d2 ? g.d1 : g.d2;
+  constexpr int kExtra = pair_extra_waves(K1::kId, K2::kId);   // a second bounded build of this pair, or 0
+  const int build = built_bound_waves(K1::kId, K2::kId, waves);
   switch (mode) {
     case MODE_HFUSE:
-      if (bounded)
+      if constexpr (kExtra != 0) {
+        if (build == kExtra) {
+          hipLaunchKernelGGL((fused_kernel_lb<K1, K2, kDlBlock, false, kExtra>), dim3(grid), dim3(g.d1 + g.d2), lds, s, x1, x2, g);
+          break;
+        }
+      }
+      if (build)
         hipLaunchKernelGGL((fused_kernel_lb<K1, K2, kDlBlock, false>), dim3(grid), dim3(g.d1 + g.d2), lds, s, x1, x2, g);
       else
         hipLaunchKernelGGL((fused_kernel<K1, K2, kDlBlock, false>), dim3(grid), dim3(g.d1 + g.d2), lds, s, x1, x2, g);
       break;
     case MODE_MATCHED:
       if constexpr (K1::kBarriers && K2::kBarriers) {
-        if (bounded)
+        if (build)
           hipLaunchKernelGGL((fused_kernel_lb<K1, K2, kDlBlock, true>), dim3(grid), dim3(g.d1 + g.d2), lds, s, x1, x2, g);
         else
           hipLaunchKernelGGL((fused_kernel<K1, K2, kDlBlock, true>), dim3(grid), dim3(g.d1 + g.d2), lds, s, x1, x2, g);
@@ -41,7 +49,7 @@ hipError_t dl_pair(FuseMode mode, bool bounded, const void *a1, const void *a2, 
       }
       break;
     case MODE_VERTICAL:
-      if (bounded)
+      if (build)   // the vertical baseline has the 8-wave bounded build only
         hipLaunchKernelGGL((vertical_kernel_lb<K1, K2, kDlBlock>), dim3(grid), dim3(wide), lds, s, x1, x2, g);
       else
         hipLaunchKernelGGL((vertical_kernel<K1, K2, kDlBlock>), dim3(grid), dim3(wide), lds, s, x1, x2, g);
@@ -54,25 +62,25 @@ hipError_t dl_pair(FuseMode mode, bool bounded, const void *a1, const void *a2, 
 }
 
 template <class K1>
-hipError_t dl_second(KernelId k2, FuseMode mode, bool bounded, const void *a1, const void *a2, const FuseGeom &g, unsigned grid,
+hipError_t dl_second(KernelId k2, FuseMode mode, int waves, const void *a1, const void *a2, const FuseGeom &g, unsigned grid,
                      size_t lds, hipStream_t s) {
   switch (k2) {
-    case K_IM2COL: return dl_pair<K1, Im2colBody>(mode, bounded, a1, a2, g, grid, lds, s);
-    case K_MAXPOOL: return dl_pair<K1, MaxPoolBody>(mode, bounded, a1, a2, g, grid, lds, s);
-    case K_BNSTATS: return dl_pair<K1, BnStatsBody>(mode, bounded, a1, a2, g, grid, lds, s);
-    case K_UPSAMPLE_NEAREST: return dl_pair<K1, UpsampleNearestBody>(mode, bounded, a1, a2, g, grid, lds, s);
-    case K_UPSAMPLE_BILINEAR: return dl_pair<K1, UpsampleBilinearBody>(mode, bounded, a1, a2, g, grid, lds, s);
-    case K_HISTC: return dl_pair<K1, HistcBody>(mode, bounded, a1, a2, g, grid, lds, s);
+    case K_IM2COL: return dl_pair<K1, Im2colBody>(mode, waves, a1, a2, g, grid, lds, s);
+    case K_MAXPOOL: return dl_pair<K1, MaxPoolBody>(mode, waves, a1, a2, g, grid, lds, s);
+    case K_BNSTATS: return dl_pair<K1, BnStatsBody>(mode, waves, a1, a2, g, grid, lds, s);
+    case K_UPSAMPLE_NEAREST: return dl_pair<K1, UpsampleNearestBody>(mode, waves, a1, a2, g, grid, lds, s);
+    case K_UPSAMPLE_BILINEAR: return dl_pair<K1, UpsampleBilinearBody>(mode, waves, a1, a2, g, grid, lds, s);
+    case K_HISTC: return dl_pair<K1, HistcBody>(mode, waves, a1, a2, g, grid, lds, s);
     default: return hipErrorNotSupported;
   }
 }
 
 // first kernel in {im2col, max-pool, batch-norm} / {upsample nearest, upsample bilinear, histogram}
-hipError_t launch_fused_dl_a(KernelId k1, KernelId k2, FuseMode mode, bool bounded, const void *a1, const void *a2,
+hipError_t launch_fused_dl_a(KernelId k1, KernelId k2, FuseMode mode, int waves, const void *a1, const void *a2,
                              const FuseGeom &g, unsigned grid, size_t lds, hipStream_t s);
-hipError_t launch_fused_dl_b(KernelId k1, KernelId k2, FuseMode mode, bool bounded, const void *a1, const void *a2,
+hipError_t launch_fused_dl_b(KernelId k1, KernelId k2, FuseMode mode, int waves, const void *a1, const void *a2,
                              const FuseGeom &g, unsigned grid, size_t lds, hipStream_t s);
-hipError_t launch_fused_dl_c(KernelId k1, KernelId k2, FuseMode mode, bool bounded, const void *a1, const void *a2,
+hipError_t launch_fused_dl_c(KernelId k1, KernelId k2, FuseMode mode, int waves, const void *a1, const void *a2,
                              const FuseGeom &g, unsigned grid, size_t lds, hipStream_t s);
 
 }  // namespace hfuse

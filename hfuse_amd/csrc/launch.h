@@ -8,20 +8,6 @@
 
 namespace hfuse {
 
-enum KernelId {
-  K_IM2COL = 0,
-  K_MAXPOOL,
-  K_BNSTATS,
-  K_UPSAMPLE_NEAREST,
-  K_HISTC,
-  K_ETHASH,
-  K_SHA256D,
-  K_SIA_BLAKE2B,
-  K_BLAKE2B,
-  K_UPSAMPLE_BILINEAR,
-  K_COUNT
-};
-
 enum FuseMode { MODE_HFUSE = 0, MODE_MATCHED = 1, MODE_BLOCKIDX = 2, MODE_VERTICAL = 3 };
 
 inline bool is_crypto(KernelId k) { return k >= K_ETHASH && k <= K_BLAKE2B; }
@@ -33,11 +19,12 @@ hipError_t launch_native_dl(KernelId k, const void *dev_args, unsigned hint, uns
 hipError_t launch_native_crypto(KernelId k, const void *dev_args, unsigned hint, unsigned grid, unsigned block,
                                 size_t lds, hipStream_t stream);
 
-// Returns hipErrorNotSupported when the pair is not instantiated.  `bounded` selects the
-// register-bounded build of the fused / vertical kernel (the launch-bound presets).
-hipError_t launch_fused_dl(KernelId k1, KernelId k2, FuseMode mode, bool bounded, const void *a1, const void *a2,
+// Returns hipErrorNotSupported when the pair is not instantiated.  `waves` selects the build of the
+// fused / vertical kernel: 0 the plain one, otherwise the register-bounded build for that many
+// waves per SIMD as built_bound_waves(k1, k2, waves) resolves it (the launch-bound presets).
+hipError_t launch_fused_dl(KernelId k1, KernelId k2, FuseMode mode, int waves, const void *a1, const void *a2,
                            const FuseGeom &g, unsigned grid, size_t lds, hipStream_t stream);
-hipError_t launch_fused_crypto(KernelId k1, KernelId k2, FuseMode mode, bool bounded, const void *a1, const void *a2,
+hipError_t launch_fused_crypto(KernelId k1, KernelId k2, FuseMode mode, int waves, const void *a1, const void *a2,
                                const FuseGeom &g, unsigned grid, size_t lds, hipStream_t stream);
 
 hipError_t launch_fill_splitmix64(unsigned long long *dst, unsigned long long nwords, unsigned long long seed,

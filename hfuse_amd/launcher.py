@@ -129,6 +129,17 @@ class Plan:
         """True / False: run the register-bounded / the plain build; None: by the preset."""
         check(L.lib().hf_plan_set_launch_bound(self._h, -1 if on is None else int(bool(on))))
 
+    def set_launch_waves(self, waves: int) -> None:
+        """Ask for the register-bounded build at `waves` waves per SIMD (1..8); 0: the occupancy formula's value."""
+        check(L.lib().hf_plan_set_launch_waves(self._h, waves))
+
+    @property
+    def launch_waves(self):
+        """(waves per SIMD the occupancy formula gives, bound of the build a launch runs now; 0 = plain)."""
+        f, b = C.c_int(), C.c_int()
+        check(L.lib().hf_plan_launch_waves(self._h, C.byref(f), C.byref(b)))
+        return f.value, b.value
+
     def bind_constants(self, constants: Optional["Constants"]) -> None:
         """Fused launches of this plan use a copy of `constants` instead of the process-wide set (None unbinds)."""
         check(L.lib().hf_plan_bind_constants(self._h, constants._h if constants is not None else None))

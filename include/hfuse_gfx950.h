@@ -191,15 +191,27 @@ HF_API int hf_plan_set_lending(hf_plan *plan, int on);
  * print `__launch_bounds__(T, B)` with B = min_k(regfile / Reg_k / size_k), capped by the
  * resident-thread limit (lib/KernelFuser/KernelPrinter.cpp:44-66), so that the compiler keeps
  * the fused kernel's registers within the occupancy the natives had.  On gfx950 that request
- * is a waves-per-SIMD bound, fixed at compile time: every pair is built twice, plain (bounded
- * only by its launch bound of 1024 or 512 threads) and register-bounded for 8 waves per SIMD
- * (at most 64 vector registers, spilling to a private stack if it must).
- *   on = 1 / 0 : run the bounded / the plain build whatever the preset;
- *   on < 0     : by the preset (default): hfuse_lb and vfuse_lb run the bounded build when
- *                launch_blocks * launch_threads asks for more than 4 waves per SIMD.
- * The blockIdx fallback has no bounded build.  Results are identical; only the time differs.
+ * is a waves-per-SIMD bound, fixed at compile time: w = B * T / 256 with this part's 128 K
+ * registers and 2048 resident threads per CU.  Every pair is built plain (bounded only by its
+ * launch bound of 1024 or 512 threads) and register-bounded for 8 waves per SIMD (at most 64
+ * vector registers, spilling to a private stack if it must); the benchmarked pairs whose formula
+ * gives less than 8 have a second bounded build at exactly their value: im2col + max-pool 5,
+ * histogram + max-pool 7, Ethash + Sia-Blake2b 6 (batch-norm + upsample and SHA-256d + Blake2b
+ * come out at 8).  A request for w waves runs the pair's own build when w is at most its value
+ * and the 8-wave build otherwise.
+ *   hf_plan_set_launch_bound: on = 1 / 0 run the bounded / the plain build whatever the preset;
+ *                on < 0 by the preset (default): hfuse_lb and vfuse_lb run the bounded build when
+ *                the formula asks for more than 4 waves per SIMD.
+ *   hf_plan_set_launch_waves: waves = 1..8 asks for a bounded build at that many waves per SIMD
+ *                (and switches the bounded build on); 0 goes back to the formula's value.
+ *   hf_plan_launch_waves: *formula = what the formula gives for this plan's block shape,
+ *                *built = the bound of the build a launch would run now (0: the plain build).
+ * The blockIdx fallback has no bounded build and the vertical baseline only the 8-wave one.
+ * Results are identical; only the time differs.
  */
 HF_API int hf_plan_set_launch_bound(hf_plan *plan, int on);
+HF_API int hf_plan_set_launch_waves(hf_plan *plan, int waves);
+HF_API int hf_plan_launch_waves(const hf_plan *plan, int *formula, int *built);
 HF_API int hf_plan_partition(const hf_plan *plan, hf_partition *out);
 /* Number of variants the reference's split loop would print (main.cpp:221-223). */
 HF_API int hf_plan_num_splits(const hf_config *cfg, int fusion_index);

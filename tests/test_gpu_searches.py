@@ -242,6 +242,31 @@ def test_every_shipped_search_pair(cuda, cfg):
     assert n == 7
 
 
+def test_ethash_sia_bounded_builds(cuda, cfg):
+    """Ethash + Sia-Blake2b in its two register-bounded builds (6 waves per SIMD, the occupancy formula's value
+    for 128 + 64 threads, and 8) against the oracle."""
+    n_items = 1 << 14
+    dag = _dag(cuda, n_items, SEED)
+    header, h2 = O.seeded_bytes(32, SEED + 30), O.seeded_bytes(80, SEED + 31)
+    target = (1 << 55) - 1
+    consts = H.Constants().set_ethash(dag, n_items, header, target).set_sia_blake2b(h2)
+    plan = cfg.plan(cfg.find_fusion("ethash_search", "sia_blake2b_gpu_hash"), "hfuse_lb")
+    plan.bind_constants(consts)
+    assert plan.launch_waves == (6, 6)
+    grid = 64
+    share = plan.partition.hi[0] - plan.partition.lo[0]
+    want1 = oracle_hits(O.ethash_search(None, SEED, n_items, header, 7, grid * share, target))
+    want2 = oracle_hits(O.sia_search(h2, 0, 1 << 15, EASY10))
+    assert want1[0] > 0 and want2[0] > 0
+    for waves in (0, 8):
+        plan.set_launch_waves(waves)
+        assert plan.launch_waves[1] == (6 if waves == 0 else 8)
+        r1, r2 = H.new_search_results(), H.new_search_results()
+        plan.launch(H.ethash_args(r1, 7), H.blake2b_args(r2, 1 << 15, 0, EASY10), grid_blocks=grid)
+        sync()
+        assert H.read_search_results(r1) == want1 and H.read_search_results(r2) == want2, waves
+
+
 def _strict(found_hits, limit, key):
     """The sub-set of an easy-target found set that also meets the stricter target `limit`."""
     hits = [h for h in found_hits[1] if key(h[1]) <= limit]

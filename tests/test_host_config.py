@@ -519,6 +519,40 @@ def test_constants_objects_are_independent_of_the_process_wide_set(cfg):
         H.Constants().set_ethash(type("T", (), {"data_ptr": lambda self: 8})(), 4, bytes(32), 1)  # misaligned DAG
 
 
+def test_launch_bound_formula_and_built_variants(cfg):
+    """The register-cap axis: the occupancy formula of the reference's printer (KernelPrinter.cpp:44-66) with
+    this part's constants, hand-worked for the five benchmarked pairs of the shipped list, and the build each
+    request resolves to.  im2col(Reg 42, 256 thr) + max-pool(32, 448): min(131072/42/256 = 12, 131072/32/448 = 9,
+    2048/704 = 2) = 2 blocks of 704 threads = 5 waves per SIMD; bn(23,128) + upsample(22,128): min(44, 46, 8) = 8
+    blocks of 256 = 8; histogram(19,768) + max-pool(32,128): min(8, 32, 2) = 2 of 896 = 7; SHA-256d(70,128) +
+    Blake2b(76,128): min(14, 13, 8) = 8 of 256 = 8; Ethash(116,128) + Blake2b(76,64): min(8, 26, 10) = 8 of 192 = 6."""
+    want = [5, 8, 7, 8, 6]
+    for i, w in enumerate(want):
+        plain, lb = cfg.plan(i), cfg.plan(i, "hfuse_lb")
+        assert plain.launch_waves == (w, 0), (i, plain.launch_waves)      # the plain preset runs the plain build
+        assert lb.launch_waves == (w, w), (i, lb.launch_waves)            # the _lb preset the pair's own bounded build
+        assert lb.partition.launch_blocks * lb.partition.launch_threads // 256 == w
+        plain.set_launch_bound(True)
+        assert plain.launch_waves == (w, w)
+        plain.set_launch_waves(8)
+        assert plain.launch_waves == (w, 8)
+        plain.set_launch_waves(3)                                         # below the pair's own value: its own build, else 8
+        assert plain.launch_waves == (w, w if w < 8 else 8)
+        plain.set_launch_waves(0)
+        plain.set_launch_bound(False)
+        assert plain.launch_waves == (w, 0)
+        with pytest.raises(hfuse_amd.HfuseError):
+            plain.set_launch_waves(9)
+        plain.set_barrier_mode(L.HF_BARRIER_BLOCKIDX)
+        plain.set_launch_bound(True)
+        assert plain.launch_waves[1] == 0                                 # the block-index partition has no bounded build
+    # pairs beyond the benchmarked five have the 8-wave build only
+    i = cfg.find_fusion("im2col_kernel", "upsample_nearest2d_out_frame")
+    p = cfg.plan(i, "hfuse_lb")
+    p.set_launch_bound(True)
+    assert p.launch_waves[1] == 8
+
+
 def test_header_symbols_are_all_exported():
     """Every function include/hfuse_gfx950.h declares is exported by the built library."""
     import os
