@@ -15,3 +15,9 @@ def default_config() -> Config:
     """The fusion list and kernel table shipped with the library."""
     return Config.from_files(os.path.join(CONFIG_DIR, "gfx950_fusion.yaml"),
                              os.path.join(CONFIG_DIR, "gfx950_kernels.yaml"))
+
+
+def triples_config() -> Config:
+    """The three-kernel fusions of the reference's lists over the same kernel table."""
+    return Config.from_files(os.path.join(CONFIG_DIR, "gfx950_triples.yaml"),
+                             os.path.join(CONFIG_DIR, "gfx950_kernels.yaml"))

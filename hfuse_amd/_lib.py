@@ -43,6 +43,15 @@ class Partition(C.Structure):
                 ("launch_blocks", C.c_uint32), ("barrier_mode", C.c_int)]
 
 
+HF_MAX_FUSE = 4
+
+
+class PartitionN(C.Structure):
+    _fields_ = [("name", C.c_char * 256), ("n", C.c_int), ("lo", C.c_uint32 * HF_MAX_FUSE), ("hi", C.c_uint32 * HF_MAX_FUSE),
+                ("block_dim", Dim3 * HF_MAX_FUSE), ("launch_threads", C.c_uint32), ("launch_blocks", C.c_uint32),
+                ("barrier_mode", C.c_int)]
+
+
 class Im2colArgs(C.Structure):
     _fields_ = [("n", C.c_int64), ("data_im", C.c_void_p)] + \
                [(k, C.c_int64) for k in ("height", "width", "kernel_h", "kernel_w", "pad_h", "pad_w",
@@ -143,6 +152,12 @@ PROTOTYPES = {
     "hf_plan_launch_waves": (C.c_int, [C.c_void_p, C.POINTER(C.c_int), C.POINTER(C.c_int)]),
     "hf_plan_set_block": (C.c_int, [C.c_void_p, C.c_int, C.c_int]),
     "hf_plan_partition": (C.c_int, [C.c_void_p, C.POINTER(Partition)]),
+    "hf_plan_num_kernels": (C.c_int, [C.c_void_p]),
+    "hf_plan_partition_n": (C.c_int, [C.c_void_p, C.POINTER(PartitionN)]),
+    "hf_plan_set_block_n": (C.c_int, [C.c_void_p, C.POINTER(C.c_int), C.c_int]),
+    "hf_launch_fused_n": (C.c_int, [C.c_void_p, C.POINTER(C.c_void_p), C.c_int, C.c_int, C.c_void_p]),
+    "hf_time_fused_n": (C.c_int, [C.c_void_p, C.c_int, C.POINTER(C.c_void_p), C.c_int, C.c_int, C.c_int, C.c_int, C.c_int,
+                                  C.c_int, C.c_void_p, C.POINTER(C.c_float)]),
     "hf_plan_num_splits": (C.c_int, [C.c_void_p, C.c_int]),
     "hf_plan_local_index": (C.c_int, [C.c_void_p, C.c_int, C.c_uint32, C.POINTER(Dim3)]),
     "hf_ethash_set_constants": (C.c_int, [C.c_void_p, C.c_uint32, C.c_char_p, C.c_uint64, C.c_void_p]),

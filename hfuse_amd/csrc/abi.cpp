@@ -559,8 +559,9 @@ struct hf_constants {
 struct hf_plan {
   bool has_consts = false;             // hf_plan_bind_constants: launches of this plan use `consts`
   SearchConstants consts;
-  KernelRow rows[2];
-  KernelId ids[2];
+  int n = 2;                           // kernels of the fusion: 2, or 3 for the reference's three-kernel lists
+  KernelRow rows[kMaxFuse];
+  KernelId ids[kMaxFuse] = {K_COUNT, K_COUNT, K_COUNT};
   const Preset *preset;
   Partition part;
   int barrier_mode;
@@ -583,6 +584,7 @@ int formula_waves(const hf_plan *plan) {
 // The launch-bound presets ask for a bounded build when the formula wants more waves per SIMD than the
 // plain build's launch bound of 1024 threads already guarantees (four).
 int plan_build_waves(const hf_plan *plan) {
+  if (plan->n != 2) return 0;  // three-kernel fusions have the plain build only
   if (!plan->preset->base_line && plan->barrier_mode == HF_BARRIER_BLOCKIDX) return 0;  // no bounded build
   const int formula = formula_waves(plan);
   const bool want = plan->bounded >= 0 ? plan->bounded != 0 : plan->preset->launch_bound && formula > 4;
@@ -591,11 +593,16 @@ int plan_build_waves(const hf_plan *plan) {
   return plan->preset->base_line ? kBoundedWaves : built;   // the vertical baseline has the 8-wave build only
 }
 
-// The reference's Context partitions a block among any number of kernels (include/KernelFusion.h:45-80;
-// configs/crypt_four.yaml fuses three); fused kernels are built for pairs here.
-int pairs_only(const FusionRow &f) {
+// The reference's Context partitions a block among any number of kernels (include/KernelFusion.h:45-80);
+// its lists hold pairs and three-kernel entries (configs/crypt_four.yaml), which is what is built here.
+int unsupported_size(const FusionRow &f) {
   return fail(HF_EUNSUPPORTED, "fusion '" + f.file + "' names " + std::to_string(f.kernels.size()) +
-                                   " kernels: fused kernels are built for pairs");
+                                   " kernels: fused kernels are built for two or three");
+}
+// Calls that shape a pair's launch (block shape, per-half grids, lending, barrier design, bounded builds).
+int pair_call_only(const hf_plan *plan) {
+  if (plan->n != 2) return fail(HF_EINVAL, "this call is for pairs; the plan fuses three kernels (see the *_n calls)");
+  return HF_OK;
 }
 }  // namespace
 
@@ -693,7 +700,8 @@ HF_API int hf_plan_num_splits(const hf_config *cfg, int fusion_index) try {
   if (!cfg) return fail(HF_EINVAL, "null config");
   if (fusion_index < 0 || fusion_index >= (int)cfg->cfg.fusions.size()) return fail(HF_EINVAL, "fusion index out of range");
   const FusionRow &f = cfg->cfg.fusions[fusion_index];
-  if (f.kernels.size() != 2) return pairs_only(f);
+  if (f.kernels.size() != 2 && f.kernels.size() != 3) return unsupported_size(f);
+  // (the driver's split loop varies the first two kernels only, main.cpp:219-225)
   return num_splits(*cfg->cfg.find(f.kernels[0]), *cfg->cfg.find(f.kernels[1]));
 } catch (...) {
   return trap_exception();
@@ -710,10 +718,11 @@ HF_API int hf_plan_create(const hf_config *cfg, int fusion_index, const char *pr
   if (split_threads > 0 && split_threads % (int)kWave != 0)
     return fail(HF_EINVAL, "split_threads must be a multiple of the 64-lane wavefront");
   const FusionRow &f = cfg->cfg.fusions[fusion_index];
-  if (f.kernels.size() != 2) return pairs_only(f);
+  if (f.kernels.size() != 2 && f.kernels.size() != 3) return unsupported_size(f);
   auto plan = new hf_plan();
   plan->preset = p;
-  for (int i = 0; i < 2; i++) {
+  plan->n = (int)f.kernels.size();
+  for (int i = 0; i < plan->n; i++) {
     plan->rows[i] = *cfg->cfg.find(f.kernels[i]);
     if (!lookup_kernel(plan->rows[i].name, plan->ids[i])) {
       int code = HF_ENOTFOUND;
@@ -721,6 +730,50 @@ HF_API int hf_plan_create(const hf_config *cfg, int fusion_index, const char *pr
       delete plan;
       return fail(code, msg);
     }
+  }
+  if (plan->n == 3) {
+    // A three-kernel list: the Context's partition among three, no tuned keys, no lending, every
+    // synchronising body on its own LDS arrival counter.
+    if (is_crypto(plan->ids[0]) != is_crypto(plan->ids[1]) || is_crypto(plan->ids[0]) != is_crypto(plan->ids[2])) {
+      delete plan;
+      return fail(HF_EUNSUPPORTED, "fusions mixing tensor kernels with search kernels are not built");
+    }
+    if (split_threads > 0) {
+      delete plan;
+      return fail(HF_EINVAL, "split_threads shapes a pair; give a three-kernel plan its block with hf_plan_set_block_n");
+    }
+    // the entry's own block shape (`Blocks:`), applied like a pair's Split / Threads: to the table split of a horizontal preset
+    KernelRow shaped[kMaxFuse] = {plan->rows[0], plan->rows[1], plan->rows[2]};
+    const bool own_shape = split_idx == HF_SPLIT_TABLE && f.blocks.size() == 3 && !p->base_line;
+    std::string label;
+    for (int i = 0; own_shape && i < 3; i++) {
+      if (shaped[i].block_dim.z != 1 || f.blocks[i] % shaped[i].block_dim.y) {
+        std::string msg = "'Blocks' entry does not divide by BlockDim.Y of '" + shaped[i].name + "'";
+        delete plan;
+        return fail(HF_EINVAL, msg);
+      }
+      shaped[i].block_dim.x = f.blocks[i] / shaped[i].block_dim.y;
+      label += "_" + std::to_string(f.blocks[i]);
+    }
+    const KernelRow *rows[kMaxFuse] = {&shaped[0], &shaped[1], &shaped[2]};
+    std::string err3;
+    int rc3 = make_partition_n(rows, 3, *p, split_idx, plan->part, err3);
+    if (rc3 == HF_OK && own_shape)
+      plan->part.name = plan->rows[0].name + "_" + plan->rows[1].name + "_" + plan->rows[2].name + "_fused_kernel_" +
+                        p->name + "_block" + label;
+    if (rc3 == HF_OK && is_crypto(plan->ids[0]) && plan->part.launch_threads > 512) {
+      rc3 = HF_EINVAL;
+      err3 = "search kernels are built for fused blocks of at most 512 threads";
+    }
+    if (rc3 != HF_OK) {
+      delete plan;
+      return fail(rc3, err3);
+    }
+    plan->lending = false;
+    plan->barrier_mode = (body_has_barriers(plan->ids[0]) || body_has_barriers(plan->ids[1]) || body_has_barriers(plan->ids[2]))
+                             ? HF_BARRIER_SUBSET : HF_BARRIER_NONE;
+    *out = plan;
+    return HF_OK;
   }
   if (is_crypto(plan->ids[0]) != is_crypto(plan->ids[1])) {
     delete plan;
@@ -771,6 +824,7 @@ HF_API int hf_plan_create(const hf_config *cfg, int fusion_index, const char *pr
 
 HF_API int hf_plan_set_barrier_mode(hf_plan *plan, int mode) try {
   if (!plan) return fail(HF_EINVAL, "null plan");
+  if (int prc = pair_call_only(plan)) return prc;
   const bool b1 = body_has_barriers(plan->ids[0]), b2 = body_has_barriers(plan->ids[1]);
   switch (mode) {
     case HF_BARRIER_NONE:
@@ -795,6 +849,7 @@ HF_API int hf_plan_set_barrier_mode(hf_plan *plan, int mode) try {
 
 HF_API int hf_plan_set_grids(hf_plan *plan, int grid1, int grid2) try {
   if (!plan) return fail(HF_EINVAL, "null plan");
+  if (int prc = pair_call_only(plan)) return prc;
   if (grid1 < 0 || grid2 < 0) return fail(HF_EINVAL, "negative grid");
   plan->grid_override[0] = (unsigned)grid1;
   plan->grid_override[1] = (unsigned)grid2;
@@ -805,6 +860,7 @@ HF_API int hf_plan_set_grids(hf_plan *plan, int grid1, int grid2) try {
 
 HF_API int hf_plan_set_block(hf_plan *plan, int threads1, int threads2) try {
   if (!plan) return fail(HF_EINVAL, "null plan");
+  if (int prc = pair_call_only(plan)) return prc;
   if (plan->preset->base_line) return fail(HF_EINVAL, "vertical presets have no thread partition to set");
   if (threads1 <= 0 || threads2 <= 0 || threads1 % (int)kWave || threads2 % (int)kWave)
     return fail(HF_EINVAL, "both parts must be positive multiples of the 64-lane wavefront");
@@ -832,6 +888,7 @@ HF_API int hf_plan_set_block(hf_plan *plan, int threads1, int threads2) try {
 
 HF_API int hf_plan_set_lending(hf_plan *plan, int on) try {
   if (!plan) return fail(HF_EINVAL, "null plan");
+  if (int prc = pair_call_only(plan)) return prc;
   plan->lending = on != 0;
   return HF_OK;
 } catch (...) {
@@ -840,6 +897,7 @@ HF_API int hf_plan_set_lending(hf_plan *plan, int on) try {
 
 HF_API int hf_plan_set_launch_bound(hf_plan *plan, int on) try {
   if (!plan) return fail(HF_EINVAL, "null plan");
+  if (int prc = pair_call_only(plan)) return prc;
   plan->bounded = on < 0 ? -1 : (on != 0);
   return HF_OK;
 } catch (...) {
@@ -848,6 +906,7 @@ HF_API int hf_plan_set_launch_bound(hf_plan *plan, int on) try {
 
 HF_API int hf_plan_set_launch_waves(hf_plan *plan, int waves) try {
   if (!plan) return fail(HF_EINVAL, "null plan");
+  if (int prc = pair_call_only(plan)) return prc;
   if (waves < 0 || waves > kBoundedWaves) return fail(HF_EINVAL, "waves per SIMD must be 0 (by the formula) or 1..8");
   plan->bound_waves = waves;
   if (waves > 0) plan->bounded = 1;
@@ -869,6 +928,7 @@ HF_API void hf_plan_free(hf_plan *plan) { delete plan; }
 
 HF_API int hf_plan_partition(const hf_plan *plan, hf_partition *out) try {
   if (!plan || !out) return fail(HF_EINVAL, "null argument");
+  if (int prc = pair_call_only(plan)) return prc;
   std::memset(out, 0, sizeof *out);
   std::strncpy(out->name, plan->part.name.c_str(), sizeof out->name - 1);
   for (int i = 0; i < 2; i++) {
@@ -884,9 +944,60 @@ HF_API int hf_plan_partition(const hf_plan *plan, hf_partition *out) try {
   return trap_exception();
 }
 
+HF_API int hf_plan_num_kernels(const hf_plan *plan) { return plan ? plan->n : fail(HF_EINVAL, "null plan"); }
+
+HF_API int hf_plan_partition_n(const hf_plan *plan, hf_partition_n *out) try {
+  if (!plan || !out) return fail(HF_EINVAL, "null argument");
+  std::memset(out, 0, sizeof *out);
+  std::strncpy(out->name, plan->part.name.c_str(), sizeof out->name - 1);
+  out->n = plan->n;
+  for (int i = 0; i < plan->n; i++) {
+    out->lo[i] = plan->part.lo[i];
+    out->hi[i] = plan->part.hi[i];
+    out->block_dim[i] = {plan->part.block_dim[i].x, plan->part.block_dim[i].y, plan->part.block_dim[i].z};
+  }
+  out->launch_threads = plan->part.launch_threads;
+  out->launch_blocks = plan->part.launch_blocks;
+  out->barrier_mode = plan->barrier_mode;
+  return HF_OK;
+} catch (...) {
+  return trap_exception();
+}
+
+HF_API int hf_plan_set_block_n(hf_plan *plan, const int *threads, int n) try {
+  if (!plan || !threads) return fail(HF_EINVAL, "null argument");
+  if (n != plan->n) return fail(HF_EINVAL, "one thread count per kernel of the plan");
+  if (plan->n == 2) return hf_plan_set_block(plan, threads[0], threads[1]);
+  if (plan->preset->base_line) return fail(HF_EINVAL, "vertical presets have no thread partition to set");
+  KernelRow rows[kMaxFuse] = {plan->rows[0], plan->rows[1], plan->rows[2]};
+  int total = 0;
+  std::string label;
+  for (int i = 0; i < n; i++) {
+    if (threads[i] <= 0 || threads[i] % (int)kWave)
+      return fail(HF_EINVAL, "every part must be a positive multiple of the 64-lane wavefront");
+    if (rows[i].block_dim.z != 1 || threads[i] % (int)rows[i].block_dim.y)
+      return fail(HF_EINVAL, "thread count does not divide by BlockDim.Y of '" + rows[i].name + "'");
+    rows[i].block_dim.x = (uint32_t)threads[i] / rows[i].block_dim.y;  // KernelFusion.h:72
+    total += threads[i];
+    label += "_" + std::to_string(threads[i]);
+  }
+  if (is_crypto(plan->ids[0]) && total > 512) return fail(HF_EINVAL, "search kernels are built for fused blocks of at most 512 threads");
+  const KernelRow *ptrs[kMaxFuse] = {&rows[0], &rows[1], &rows[2]};
+  Partition part;
+  std::string err;
+  int rc = make_partition_n(ptrs, n, *plan->preset, HF_SPLIT_TABLE, part, err);
+  if (rc != HF_OK) return fail(rc, err);
+  part.name = plan->rows[0].name + "_" + plan->rows[1].name + "_" + plan->rows[2].name + "_fused_kernel_" +
+              plan->preset->name + "_block" + label;
+  plan->part = part;
+  return HF_OK;
+} catch (...) {
+  return trap_exception();
+}
+
 HF_API int hf_plan_local_index(const hf_plan *plan, int half, uint32_t tid, hf_dim3 *out) try {
   if (!plan || !out) return fail(HF_EINVAL, "null argument");
-  if (half < 0 || half > 1) return fail(HF_EINVAL, "half must be 0 or 1");
+  if (half < 0 || half >= plan->n) return fail(HF_EINVAL, "kernel index outside the plan");
   if (tid < plan->part.lo[half] || tid >= plan->part.hi[half])
     return fail(HF_EINVAL, "thread is outside this kernel's bounds");
   Dim3 d = local_index(tid, plan->part.lo[half], plan->part.block_dim[half]);
@@ -1153,6 +1264,7 @@ int do_launch_fused(const hf_plan *plan, const Prepared &p1, const Prepared &p2,
 
 HF_API int hf_launch_fused(const hf_plan *plan, const void *args1, const void *args2, int grid_blocks, void *stream) try {
   if (!plan) return fail(HF_EINVAL, "null plan");
+  if (int prc = pair_call_only(plan)) return prc;
   Prepared p1, p2;
   const SearchConstants *consts = plan->has_consts ? &plan->consts : nullptr;
   int rc = prepare(plan->ids[0], args1, p1, consts);
@@ -1167,6 +1279,7 @@ HF_API int hf_launch_fused(const hf_plan *plan, const void *args1, const void *a
 HF_API int hf_time_pair(const hf_plan *plan, int mode, const void *const *args1, const void *const *args2, int nsets,
                         int first_set, int warmup, int iters, int grid_blocks, void *stream_, float *elapsed_ms) try {
   if (!plan || !args1 || !args2 || !elapsed_ms) return fail(HF_EINVAL, "null argument");
+  if (int prc = pair_call_only(plan)) return prc;
   if (nsets <= 0 || iters <= 0 || warmup < 0 || mode < 0 || mode > 4 || first_set < 0 || first_set >= nsets)
     return fail(HF_EINVAL, "bad repetition arguments");
   hipStream_t stream = static_cast<hipStream_t>(stream_);
@@ -1235,6 +1348,101 @@ HF_API int hf_time_pair(const hf_plan *plan, int mode, const void *const *args1,
   int rc = HF_OK;
   e = hipEventRecord(t0, stream);
   for (int i = 0; i < iters && rc == HF_OK && e == hipSuccess; i++) rc = once(warmup + i);
+  if (e == hipSuccess) e = hipEventRecord(t1, stream);
+  if (e == hipSuccess) e = hipEventSynchronize(t1);
+  if (e == hipSuccess) e = hipEventElapsedTime(elapsed_ms, t0, t1);
+  (void)hipEventDestroy(t0);
+  (void)hipEventDestroy(t1);
+  if (rc != HF_OK) return rc;
+  if (e != hipSuccess) return hip_fail(e, "timing");
+  return HF_OK;
+} catch (...) {
+  return trap_exception();
+}
+
+namespace {
+
+int do_launch_fused3(const hf_plan *plan, const Prepared *p, int grid_blocks, hipStream_t stream) {
+  FuseGeom3 g;
+  const bool vertical = plan->preset->base_line;
+  unsigned block = 0, grid = 0;
+  size_t lds = 4 * kBarrierWords;
+  for (int i = 0; i < 3; i++) {
+    g.d[i] = plan->part.hi[i] - plan->part.lo[i];
+    g.lds[i] = (p[i].lds + 15u) & ~15u;
+    g.hint[i] = p[i].hint;
+    lds += g.lds[i];
+    block = vertical ? std::max(block, g.d[i]) : block + g.d[i];
+  }
+  for (int i = 0; i < 3; i++) {
+    if (grid_blocks > 0) g.grid[i] = (unsigned)grid_blocks;
+    else g.grid[i] = p[i].exact_grid ? kDefaultEthashGrid : (p[i].items == 0 ? 0u : default_grid(p[i], g.d[i], block));
+    grid = std::max(grid, g.grid[i]);
+  }
+  if (grid == 0) return HF_OK;  // nothing to do
+  const unsigned long long threads = (unsigned long long)grid * block;
+  if (threads > 0xFFFFFFFFull || !counter_fits(p[0], threads) || !counter_fits(p[1], threads) || !counter_fits(p[2], threads))
+    return fail(HF_EINVAL, kCounterMsg);
+  const void *const blobs[3] = {p[0].blob, p[1].blob, p[2].blob};
+  const hipError_t e = is_crypto(plan->ids[0]) ? launch_fused3_crypto(plan->ids, vertical, blobs, g, grid, block, lds, stream)
+                                               : launch_fused3_dl(plan->ids, vertical, blobs, g, grid, block, lds, stream);
+  if (e == hipErrorNotSupported) return fail(HF_EUNSUPPORTED, "this three-kernel list is not built (built: the reference's lists, in their order)");
+  if (e != hipSuccess) return hip_fail(e, "fused launch");
+  return HF_OK;
+}
+
+}  // namespace
+
+HF_API int hf_launch_fused_n(const hf_plan *plan, const void *const *args, int n, int grid_blocks, void *stream) try {
+  if (!plan || !args) return fail(HF_EINVAL, "null argument");
+  if (n != plan->n) return fail(HF_EINVAL, "one argument list per kernel of the plan");
+  if (n == 2) return hf_launch_fused(plan, args[0], args[1], grid_blocks, stream);
+  Prepared p[3];
+  const SearchConstants *consts = plan->has_consts ? &plan->consts : nullptr;
+  for (int i = 0; i < 3; i++) {
+    int rc = prepare(plan->ids[i], args[i], p[i], consts);
+    if (rc != HF_OK) return rc;
+  }
+  return do_launch_fused3(plan, p, grid_blocks, static_cast<hipStream_t>(stream));
+} catch (...) {
+  return trap_exception();
+}
+
+HF_API int hf_time_fused_n(const hf_plan *plan, int mode, const void *const *args, int n, int nsets, int first_set,
+                           int warmup, int iters, int grid_blocks, void *stream_, float *elapsed_ms) try {
+  if (!plan || !args || !elapsed_ms) return fail(HF_EINVAL, "null argument");
+  if (n != plan->n || n != 3) return fail(HF_EINVAL, "hf_time_fused_n times three-kernel plans (pairs: hf_time_pair)");
+  if (nsets <= 0 || iters <= 0 || warmup < 0 || (mode != 2 && mode != 3) || first_set < 0 || first_set >= nsets)
+    return fail(HF_EINVAL, "bad repetition arguments");
+  hipStream_t stream = static_cast<hipStream_t>(stream_);
+  const SearchConstants *consts = plan->has_consts ? &plan->consts : nullptr;
+  std::vector<Prepared> p((size_t)nsets * 3);
+  for (int s = 0; s < nsets; s++)
+    for (int i = 0; i < 3; i++) {
+      int rc = prepare(plan->ids[i], args[(size_t)s * 3 + i], p[(size_t)s * 3 + i], consts);
+      if (rc != HF_OK) return rc;
+    }
+  auto once = [&](int r) -> int {
+    const Prepared *q = &p[(size_t)(((long long)first_set + r) % nsets) * 3];
+    if (mode == 3) return do_launch_fused3(plan, q, grid_blocks, stream);
+    for (int i = 0; i < 3; i++) {
+      int rc = do_launch_native(plan->ids[i], q[i], q[i].exact_grid ? grid_blocks : 0, plan->rows[i].native_block(), stream);
+      if (rc != HF_OK) return rc;
+    }
+    return HF_OK;
+  };
+  for (int r = 0; r < warmup; r++) {
+    int rc = once(r);
+    if (rc != HF_OK) return rc;
+  }
+  hipEvent_t t0, t1;
+  hipError_t e = hipEventCreate(&t0);
+  if (e != hipSuccess) return hip_fail(e, "hipEventCreate");
+  e = hipEventCreate(&t1);
+  if (e != hipSuccess) { (void)hipEventDestroy(t0); return hip_fail(e, "hipEventCreate"); }
+  int rc = HF_OK;
+  e = hipEventRecord(t0, stream);
+  for (int r = 0; r < iters && rc == HF_OK && e == hipSuccess; r++) rc = once(warmup + r);
   if (e == hipSuccess) e = hipEventRecord(t1, stream);
   if (e == hipSuccess) e = hipEventSynchronize(t1);
   if (e == hipSuccess) e = hipEventElapsedTime(elapsed_ms, t0, t1);

@@ -273,4 +273,71 @@ void vertical_kernel_lb(typename K1::Args a1, typename K2::Args a2, FuseGeom g) 
   vertical_block<K1, K2>(a1, a2, g);
 }
 
+// ----------------------------------------------------------------------------
+// Three kernels in one workgroup (the reference's Context partitions a block among any number of
+// kernels, include/KernelFusion.h:45-80; configs/crypt_four.yaml and im2col_maxpool_norm.yaml
+// list three).  Waves [0, d0/64) run kernel 0, the next d1/64 kernel 1, the rest kernel 2.  Each
+// kernel strides over its own number of workgroups; in a block beyond that number its waves end at
+// once (no lending here).  A body that synchronises uses its own LDS arrival counter.
+// ----------------------------------------------------------------------------
+struct FuseGeom3 {
+  unsigned d[3];     // threads of each part
+  unsigned lds[3];   // LDS bytes of each part
+  unsigned hint[3];  // fast-path selectors
+  unsigned grid[3];  // workgroups each kernel strides over
+};
+
+template <class K, int BAR>
+__device__ __forceinline__ void run_part(const typename K::Args &a, unsigned tid, unsigned d, unsigned bid, unsigned grid,
+                                         unsigned *bar, unsigned char *lds, unsigned hint) {
+  if (bid >= grid) return;
+  SubBlock<BAR> sb{tid, d, bid, grid, bar, 0, bid * d, grid * d};
+  K::run(a, sb, lds, hint);
+}
+
+template <class K0, class K1, class K2, int T>
+__global__ __launch_bounds__(T) void fused_kernel3(typename K0::Args a0, typename K1::Args a1, typename K2::Args a2,
+                                                   FuseGeom3 g) {
+  extern __shared__ __align__(16) unsigned char smem[];
+  unsigned *bars = reinterpret_cast<unsigned *>(smem);
+  const unsigned tid = threadIdx.x, bid = blockIdx.x;
+  constexpr bool kAny = K0::kBarriers || K1::kBarriers || K2::kBarriers;
+  if constexpr (kAny) {
+    if (tid < kBarrierWords) bars[tid] = 0;
+    __syncthreads();
+  }
+  const unsigned wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const unsigned w0 = g.d[0] >> 6, w1 = w0 + (g.d[1] >> 6);
+  unsigned char *l0 = smem + 4 * kBarrierWords, *l1 = l0 + g.lds[0], *l2 = l1 + g.lds[1];
+  if (wave < w0)
+    run_part<K0, K0::kBarriers ? BAR_SUBSET : BAR_WORKGROUP>(a0, tid, g.d[0], bid, g.grid[0], bars + 0, l0, g.hint[0]);
+  else if (wave < w1)
+    run_part<K1, K1::kBarriers ? BAR_SUBSET : BAR_WORKGROUP>(a1, tid - g.d[0], g.d[1], bid, g.grid[1], bars + 1, l1, g.hint[1]);
+  else
+    run_part<K2, K2::kBarriers ? BAR_SUBSET : BAR_WORKGROUP>(a2, tid - g.d[0] - g.d[1], g.d[2], bid, g.grid[2], bars + 2, l2,
+                                                             g.hint[2]);
+}
+
+// The vertical baseline of a three-kernel list: a block of max(d) threads runs the bodies one after the other.
+template <class K0, class K1, class K2, int T>
+__global__ __launch_bounds__(T) void vertical_kernel3(typename K0::Args a0, typename K1::Args a1, typename K2::Args a2,
+                                                      FuseGeom3 g) {
+  extern __shared__ __align__(16) unsigned char smem[];
+  unsigned *bars = reinterpret_cast<unsigned *>(smem);
+  const unsigned tid = threadIdx.x, bid = blockIdx.x;
+  constexpr bool kAny = K0::kBarriers || K1::kBarriers || K2::kBarriers;
+  if constexpr (kAny) {
+    if (tid < kBarrierWords) bars[tid] = 0;
+    __syncthreads();
+  }
+  const unsigned wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  unsigned char *l0 = smem + 4 * kBarrierWords, *l1 = l0 + g.lds[0], *l2 = l1 + g.lds[1];
+  if (wave < (g.d[0] >> 6))
+    run_part<K0, K0::kBarriers ? BAR_SUBSET : BAR_WORKGROUP>(a0, tid, g.d[0], bid, g.grid[0], bars + 0, l0, g.hint[0]);
+  if (wave < (g.d[1] >> 6))
+    run_part<K1, K1::kBarriers ? BAR_SUBSET : BAR_WORKGROUP>(a1, tid, g.d[1], bid, g.grid[1], bars + 1, l1, g.hint[1]);
+  if (wave < (g.d[2] >> 6))
+    run_part<K2, K2::kBarriers ? BAR_SUBSET : BAR_WORKGROUP>(a2, tid, g.d[2], bid, g.grid[2], bars + 2, l2, g.hint[2]);
+}
+
 }  // namespace hfuse

@@ -190,9 +190,24 @@ bool parse_config(const char *fusion_yaml, const char *kernels_yaml, Config &cfg
           return false;
         }
       }
+      if (const YamlNode *bl = n.get("Blocks")) {
+        // not in the reference's schema: the block shape of a three-kernel entry, one thread count per kernel
+        if (bl->kind != YamlNode::Seq || bl->seq.size() != ks->seq.size() || ks->seq.size() != 3) {
+          err = "fusion list: " + at(*bl) + "'Blocks' must list one thread count per kernel of a three-kernel entry";
+          return false;
+        }
+        for (auto &b : bl->seq) {
+          uint32_t t = 0;
+          if (!to_uint(&b, t) || t == 0 || t % kWave != 0 || t > kMaxBlock) {
+            err = "fusion list: " + at(b) + "'Blocks' entries must be multiples of 64 between 64 and 1024";
+            return false;
+          }
+          f.blocks.push_back(t);
+        }
+      }
       for (auto &kv : n.map)
         if (kv.first != "File" && kv.first != "Kernels" && kv.first != "Split" && kv.first != "Threads" &&
-            kv.first != "Lending" && kv.first != "Barrier" && kv.first != "LaunchBound") {
+            kv.first != "Lending" && kv.first != "Barrier" && kv.first != "LaunchBound" && kv.first != "Blocks") {
           err = "fusion list: " + at(kv.second) + "unknown key '" + kv.first + "'";
           return false;
         }
@@ -306,6 +321,89 @@ int make_partition(const KernelRow &k1, const KernelRow &k2, const Preset &prese
   out.launch_blocks = preset.launch_bound ? max_block : 0;
   out.bound_blocks = max_block;
   out.name = k1.name + "_" + k2.name + "_fused_kernel_" + variant;  // KernelPrinter.cpp:67-70
+  return HF_OK;
+}
+
+int make_partition_n(const KernelRow *const *rows, int n, const Preset &preset, int split_idx, Partition &out,
+                     std::string &err) {
+  if (n < 2 || n > kMaxFuse) { err = "a fused kernel holds two or three kernels"; return HF_EUNSUPPORTED; }
+  Dim3 dims[kMaxFuse];
+  uint32_t total = 0;
+  for (int i = 0; i < n; i++) {
+    dims[i] = rows[i]->block_dim;
+    if (dims[i].size() == 0) { err = "empty BlockDim"; return HF_EINVAL; }
+    total += dims[i].size();
+  }
+  std::string variant = preset.name;
+  if (!preset.base_line && (split_idx >= 0 || split_idx == HF_SPLIT_EXECTIME)) {
+    // Context's imbalanced re-split (KernelFusion.h:53-72) with the wavefront as granule.
+    double e[kMaxFuse], total_time = 0.0;
+    for (int i = 0; i < n; i++) e[i] = rows[i]->exec_time;
+    if (split_idx >= 0) {
+      const uint32_t end = dims[0].size() + dims[1].size();  // main.cpp:219-225: only the first two vary
+      uint32_t count = 0;
+      for (uint32_t split = 128; split < end; split += 128) count++;
+      if ((uint32_t)split_idx >= count) { err = "split index beyond the enumeration 128*(n+1) < d1+d2"; return HF_EINVAL; }
+      e[0] = 128.0 * (split_idx + 1);
+      e[1] = (double)end - e[0];
+      variant += "_idx_" + std::to_string(split_idx);
+    } else {
+      for (int i = 0; i < n; i++)
+        if (!(e[i] > 0)) { err = "ExecTime split requested but the table has no ExecTime"; return HF_EINVAL; }
+      variant += "_exectime";
+    }
+    for (int i = 0; i < n; i++) total_time += e[i];
+    if (!(total_time > 0)) { err = "ExecTimes do not sum to a positive time"; return HF_EINVAL; }
+    uint32_t allocated = 0;
+    for (int i = 0; i < n; i++) {
+      uint32_t part;
+      if (i == n - 1) {
+        if (allocated >= total) { err = "split leaves one kernel without threads"; return HF_EINVAL; }
+        part = total - allocated;
+      } else {
+        const double share = e[i] / total_time * total / kWave;
+        if (!(share >= 1.0) || share > 1e6) { err = "split leaves one kernel without threads"; return HF_EINVAL; }
+        part = (uint32_t)((int)share) * kWave;
+        allocated += part;
+      }
+      if (dims[i].z != 1 || part % dims[i].y != 0) {
+        err = "split of " + std::to_string(part) + " threads does not divide by BlockDim.Y of '" + rows[i]->name + "'";
+        return HF_EINVAL;
+      }
+      dims[i].x = part / dims[i].y;  // KernelFusion.h:72
+    }
+  } else if (!preset.base_line) {
+    variant += "_table";
+  } else {
+    variant += "_idx_0";
+  }
+  uint32_t sum = 0, max_thread = 0, max_block = 9999999u, b = 0;
+  for (int i = 0; i < n; i++) {
+    const uint32_t size = dims[i].size();
+    if (size == 0 || size % kWave != 0) {
+      err = "part of '" + rows[i]->name + "' is " + std::to_string(size) + " threads: not a multiple of the 64-lane wavefront";
+      return HF_EINVAL;
+    }
+    out.lo[i] = b;
+    out.hi[i] = b + size;
+    out.block_dim[i] = dims[i];
+    if (!preset.base_line) b += size;  // KernelFusion.h:76-78
+    if (rows[i]->reg) max_block = std::min(kRegFile / rows[i]->reg / size, max_block);  // KernelPrinter.cpp:46-60
+    sum += size;
+    max_thread = std::max(max_thread, size);
+  }
+  if ((preset.base_line ? max_thread : sum) > kMaxBlock) {
+    err = "fused block of " + std::to_string(preset.base_line ? max_thread : sum) + " threads exceeds 1024";
+    return HF_EINVAL;
+  }
+  max_block = std::min(max_block, kMaxResidentThreads / sum);
+  out.n = n;
+  out.launch_threads = preset.base_line ? max_thread : sum;
+  out.launch_blocks = preset.launch_bound ? max_block : 0;
+  out.bound_blocks = max_block;
+  out.name.clear();
+  for (int i = 0; i < n; i++) out.name += rows[i]->name + "_";  // KernelPrinter.cpp:67-70
+  out.name += "fused_kernel_" + variant;
   return HF_OK;
 }
 

@@ -35,6 +35,7 @@ struct FusionRow {
   int lending = -1;      // optional `Lending:` key: 0 / 1 switch wave lending off / on, -1 = library default
   int launch_bound = -1; // optional `LaunchBound:` key: 0 / 1 pick the plain / register-bounded build, -1 = the preset's
   int barrier = -1;      // optional `Barrier:` key: an HF_BARRIER_* mode, -1 = library default
+  std::vector<uint32_t> blocks;  // optional `Blocks:` key of a three-kernel entry: threads of each kernel in the fused block
 };
 
 struct Config {
@@ -50,9 +51,12 @@ struct Preset {
 };
 const Preset *find_preset(const std::string &name);
 
+constexpr int kMaxFuse = 3;  // kernels in one fused kernel: pairs, and the three-kernel lists of the reference
+
 struct Partition {
-  uint32_t lo[2], hi[2];
-  Dim3 block_dim[2];
+  int n = 2;  // kernels partitioned
+  uint32_t lo[kMaxFuse] = {0, 0, 0}, hi[kMaxFuse] = {0, 0, 0};
+  Dim3 block_dim[kMaxFuse];
   uint32_t launch_threads = 0, launch_blocks = 0;
   uint32_t bound_blocks = 0;  // the printer's min-blocks value whatever the preset (launch_blocks is 0 without LaunchBound)
   std::string name;  // <K1>_<K2>_fused_kernel_<preset>_idx_<n>
@@ -75,6 +79,15 @@ int num_splits(const KernelRow &k1, const KernelRow &k2);
 // Returns 0, or a negative HF_E* code with `err` set.
 int make_partition(const KernelRow &k1, const KernelRow &k2, const Preset &preset, int split_idx,
                    int split_threads, Partition &out, std::string &err);
+
+// The same for a fusion of `n` kernels (the Context partitions a block among any number,
+// include/KernelFusion.h:45-80; the driver's split loop still varies only the first two,
+// main.cpp:215-227, the others keep the table's ExecTime, -1 when the row has none).
+//   split_idx >= 0: ExecTime_0 = 128*(idx+1), ExecTime_1 = (d_0 + d_1) - ExecTime_0, then the re-split
+//   in proportion to all ExecTimes, each part rounded down to whole wavefronts, the last takes the rest;
+//   HF_SPLIT_EXECTIME: the same with the table's ExecTimes; HF_SPLIT_TABLE: the table's BlockDims.
+int make_partition_n(const KernelRow *const *rows, int n, const Preset &preset, int split_idx, Partition &out,
+                     std::string &err);
 
 // ThreadInfoRewriter.cpp:38-58
 Dim3 local_index(uint32_t tid, uint32_t lo, const Dim3 &dim);

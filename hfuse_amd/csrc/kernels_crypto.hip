@@ -74,6 +74,23 @@ hipError_t launch_native_crypto(KernelId k, const void *args, unsigned hint, uns
   }
 }
 
+// The three-kernel list of configs/crypt_four.yaml, in its listed order.
+hipError_t launch_fused3_crypto(const KernelId k[3], bool vertical, const void *const a[3], const FuseGeom3 &g, unsigned grid,
+                                unsigned block, size_t lds, hipStream_t s) {
+  if (!(k[0] == K_BLAKE2B && k[1] == K_SHA256D && k[2] == K_ETHASH)) return hipErrorNotSupported;
+  if (block > (unsigned)kCryptoBlock) return hipErrorNotSupported;
+  const auto &x0 = *static_cast<const Blake2bDevArgs *>(a[0]);
+  const auto &x1 = *static_cast<const Sha256dDevArgs *>(a[1]);
+  const auto &x2 = *static_cast<const EthashDevArgs *>(a[2]);
+  if (vertical)
+    hipLaunchKernelGGL((vertical_kernel3<CcminerBlake2bBody, Sha256dBody, EthashBody, kCryptoBlock>), dim3(grid), dim3(block),
+                       lds, s, x0, x1, x2, g);
+  else
+    hipLaunchKernelGGL((fused_kernel3<CcminerBlake2bBody, Sha256dBody, EthashBody, kCryptoBlock>), dim3(grid), dim3(block), lds,
+                       s, x0, x1, x2, g);
+  return hipGetLastError();
+}
+
 #define HF_PAIR(A, KA, B, KB)                                                     \
   if (k1 == A && k2 == B) return pair<KA, KB>(mode, waves, a1, a2, g, grid, lds, s);     \
   if (k1 == B && k2 == A) return pair<KB, KA>(mode, waves, a1, a2, g, grid, lds, s);

@@ -27,6 +27,12 @@ hipError_t launch_fused_dl(KernelId k1, KernelId k2, FuseMode mode, int waves, c
 hipError_t launch_fused_crypto(KernelId k1, KernelId k2, FuseMode mode, int waves, const void *a1, const void *a2,
                                const FuseGeom &g, unsigned grid, size_t lds, hipStream_t stream);
 
+// Three-kernel fusions (vertical = the baseline preset).  hipErrorNotSupported when the list is not instantiated.
+hipError_t launch_fused3_dl(const KernelId k[3], bool vertical, const void *const a[3], const FuseGeom3 &g, unsigned grid,
+                            unsigned block, size_t lds, hipStream_t stream);
+hipError_t launch_fused3_crypto(const KernelId k[3], bool vertical, const void *const a[3], const FuseGeom3 &g, unsigned grid,
+                                unsigned block, size_t lds, hipStream_t stream);
+
 hipError_t launch_fill_splitmix64(unsigned long long *dst, unsigned long long nwords, unsigned long long seed,
                                   hipStream_t stream);
 hipError_t launch_copy_f32(const float *src, float *dst, unsigned long long n, hipStream_t stream);

@@ -70,6 +70,13 @@ class Config:
             out.append(name.value.decode())
         return out
 
+    def find_fusion_n(self, *kernels: str) -> int:
+        """Index of the entry that lists exactly these kernels in this order (any number of them)."""
+        for i in range(self.num_fusions):
+            if self.fusion_kernels(i) == list(kernels):
+                return i
+        raise KeyError(f"no fusion of {' + '.join(kernels)} in the fusion list")
+
     def find_fusion(self, k1: str, k2: str) -> int:
         for i, (_, a, b) in enumerate(self.fusions()):
             if (a, b) == (k1, k2) and check(L.lib().hf_config_fusion_size(self._h, i)) == 2:
@@ -112,6 +119,38 @@ class Plan:
     @property
     def name(self) -> str:
         return self.partition.name.decode()
+
+    @property
+    def num_kernels(self) -> int:
+        return check(L.lib().hf_plan_num_kernels(self._h))
+
+    @property
+    def partition_n(self) -> L.PartitionN:
+        out = L.PartitionN()
+        check(L.lib().hf_plan_partition_n(self._h, C.byref(out)))
+        return out
+
+    def set_block_n(self, *threads: int) -> None:
+        arr = (C.c_int * len(threads))(*threads)
+        check(L.lib().hf_plan_set_block_n(self._h, arr, len(threads)))
+
+    def launch_n(self, args: Sequence, grid_blocks: int = 0, stream=None) -> None:
+        """Fused launch of a plan of len(args) kernels, argument lists in YAML order."""
+        ptrs = (C.c_void_p * len(args))(*[C.addressof(a) for a in args])
+        check(L.lib().hf_launch_fused_n(self._h, ptrs, len(args), grid_blocks, _stream_ptr(stream)))
+
+    def time_n(self, mode: int, arg_sets: Sequence[Sequence], warmup: int, iters: int, grid_blocks: int = 0,
+               stream=None, rotation: Optional["Rotation"] = None) -> float:
+        """Milliseconds for `iters` repetitions of a three-kernel plan (mode 2 natives back to back, 3 fused);
+        arg_sets[s][k] is kernel k's argument list of buffer set s."""
+        nsets, n = len(arg_sets), len(arg_sets[0])
+        flat = [C.addressof(a) for s in arg_sets for a in s]
+        ptrs = (C.c_void_p * len(flat))(*flat)
+        ms = C.c_float()
+        first = rotation.take(nsets, warmup + iters) if rotation is not None else 0
+        check(L.lib().hf_time_fused_n(self._h, mode, ptrs, n, nsets, first, warmup, iters, grid_blocks,
+                                      _stream_ptr(stream), C.byref(ms)))
+        return ms.value
 
     def set_barrier_mode(self, mode: int) -> None:
         check(L.lib().hf_plan_set_barrier_mode(self._h, mode))

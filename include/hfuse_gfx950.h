@@ -99,8 +99,8 @@ HF_API int hf_config_num_kernels(const hf_config *cfg);
  * Names of the i-th fusion's kernels (NUL-terminated, valid while cfg lives).  The schema lets an
  * entry name any number of kernels (include/KernelFusion.h:140-146; configs/crypt_four.yaml names
  * three): such a list loads, hf_config_fusion gives its first two names (k2 = "" for a single one),
- * hf_config_fusion_size / hf_config_fusion_kernel give all of them, and hf_plan_create answers
- * HF_EUNSUPPORTED for every entry that is not a pair.
+ * hf_config_fusion_size / hf_config_fusion_kernel give all of them.  Plans exist for entries of two
+ * and of three kernels; hf_plan_create answers HF_EUNSUPPORTED for any other size.
  */
 HF_API int hf_config_fusion(const hf_config *cfg, int i, const char **file, const char **k1,
                             const char **k2);
@@ -213,6 +213,40 @@ HF_API int hf_plan_set_launch_bound(hf_plan *plan, int on);
 HF_API int hf_plan_set_launch_waves(hf_plan *plan, int waves);
 HF_API int hf_plan_launch_waves(const hf_plan *plan, int *formula, int *built);
 HF_API int hf_plan_partition(const hf_plan *plan, hf_partition *out);
+/*
+ * Three-kernel fusions.  The reference's Context partitions one block among any number of kernels
+ * (include/KernelFusion.h:45-80) and its lists name three in configs/crypt_four.yaml
+ * (blake2b_gpu_hash, sha256d_gpu_hash_shared, ethash_search4), configs/im2col_maxpool_norm.yaml
+ * and configs/maxpool_summary_norm.yaml; those three lists are built, in their listed order.
+ * hf_plan_create on such an entry gives a plan whose block is kernel 0's threads, then kernel
+ * 1's, then kernel 2's (vfuse presets: all three start at thread 0 of a block of max threads).
+ *   split_idx     : as the reference's driver does it (main.cpp:215-227): only the first two
+ *                   kernels' ExecTimes are varied, ExecTime_0 = 128*(idx+1), ExecTime_1 =
+ *                   (d0 + d1) - ExecTime_0, the third keeps the table's (-1 without the key); the
+ *                   Context then re-splits d0 + d1 + d2 in proportion, whole wavefronts each,
+ *                   the last kernel taking the rest.  HF_SPLIT_EXECTIME / HF_SPLIT_TABLE as for pairs.
+ *   split_threads : must be 0; hf_plan_set_block_n shapes the block freely.
+ * Each kernel strides over its own number of workgroups (the launch covers the largest); in a
+ * block beyond a kernel's own number its wavefronts end at once.  A body that synchronises does
+ * so on its own LDS arrival counter.  The calls that shape a pair (hf_plan_set_block / _grids /
+ * _lending / _barrier_mode / _launch_bound / _launch_waves, hf_plan_partition, hf_launch_fused,
+ * hf_time_pair) answer HF_EINVAL for a three-kernel plan; hf_plan_bind_constants and
+ * hf_plan_local_index (half = 0..2) apply.
+ */
+#define HF_MAX_FUSE 4
+typedef struct {
+  char name[256];                /* <K0>_<K1>_<K2>_fused_kernel_<preset>_idx_<n>    */
+  int n;                         /* kernels in the plan: 2 or 3                      */
+  uint32_t lo[HF_MAX_FUSE], hi[HF_MAX_FUSE];
+  hf_dim3 block_dim[HF_MAX_FUSE];
+  uint32_t launch_threads, launch_blocks;
+  int barrier_mode;
+} hf_partition_n;
+HF_API int hf_plan_num_kernels(const hf_plan *plan);
+HF_API int hf_plan_partition_n(const hf_plan *plan, hf_partition_n *out);
+/* threads[k] for kernel k (multiples of 64 that divide by its BlockDim.Y; sum <= 1024, 512 for the searches). */
+HF_API int hf_plan_set_block_n(hf_plan *plan, const int *threads, int n);
+
 /* Number of variants the reference's split loop would print (main.cpp:221-223). */
 HF_API int hf_plan_num_splits(const hf_config *cfg, int fusion_index);
 /* Local (x,y,z) of flat thread `tid` in half `half`: ThreadInfoRewriter.cpp:38-58. */
@@ -425,6 +459,20 @@ HF_API int hf_launch_native_with(const char *kernel_name, const void *args,
  */
 HF_API int hf_launch_fused(const hf_plan *plan, const void *args1, const void *args2,
                            int grid_blocks, void *stream);
+
+/*
+ * Fused launch of a plan of n kernels: args[k] points at kernel k's argument list, in YAML order
+ * (n = 2 is hf_launch_fused).  grid_blocks > 0: every kernel strides over that many workgroups.
+ */
+HF_API int hf_launch_fused_n(const hf_plan *plan, const void *const *args, int n, int grid_blocks,
+                             void *stream);
+/*
+ * hf_time_pair for a three-kernel plan: mode 2 = the three native kernels back to back on
+ * `stream`, mode 3 = the fused kernel; args[s * n + k] is kernel k's argument list of set s.
+ */
+HF_API int hf_time_fused_n(const hf_plan *plan, int mode, const void *const *args, int n, int nsets,
+                           int first_set, int warmup, int iters, int grid_blocks, void *stream,
+                           float *elapsed_ms);
 
 /*
  * Timing helper used by the benchmark: runs `iters` repetitions of

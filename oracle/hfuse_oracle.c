@@ -138,6 +138,65 @@ ORC_API int orc_context(const orc_kernel_info *k, int base_line, int launch_boun
 }
 
 /*
+ * The same Context constructor for a list of n kernels (include/KernelFusion.h:45-80 loops over all
+ * Infos; configs/crypt_four.yaml, im2col_maxpool_norm.yaml and maxpool_summary_norm.yaml list three):
+ * with `imbalanced`, kernel i < n-1 gets int(ExecTime_i / sum(ExecTime) * sum(threads) / granule) * granule
+ * threads and the last one the rest; bounds are consecutive unless base_line.  Launch bounds as above,
+ * the minimum and the sums running over all n kernels (KernelPrinter.cpp:46-60).
+ */
+#define ORC_MAX_FUSE 4
+typedef struct {
+  uint32_t lo[ORC_MAX_FUSE], hi[ORC_MAX_FUSE];
+  orc_dim3 block_dim[ORC_MAX_FUSE];
+  uint32_t launch_threads, launch_blocks;
+} orc_partition_n;
+
+ORC_API int orc_context_n(const orc_kernel_info *k, int n, int base_line, int launch_bound, int imbalanced,
+                          uint32_t granule, uint32_t reg_file, uint32_t max_threads, orc_partition_n *out) {
+  if (n < 1 || n > ORC_MAX_FUSE) return -1;
+  double total_time = 0.0;
+  uint32_t total_thread = 0, allocated = 0, b = 0;
+  orc_dim3 dims[ORC_MAX_FUSE];
+  for (int i = 0; i < n; i++) {
+    total_time += k[i].exec_time;
+    total_thread += k[i].block_dim.x * k[i].block_dim.y * k[i].block_dim.z;
+  }
+  for (int i = 0; i < n; i++) {
+    dims[i] = k[i].block_dim;
+    if (imbalanced) {
+      uint32_t thread;
+      if (i == n - 1) {
+        thread = total_thread - allocated;
+      } else {
+        thread = (uint32_t)((int)(k[i].exec_time / total_time * total_thread / granule)) * granule;
+        allocated += thread;
+      }
+      dims[i].x = thread / dims[i].y;
+    }
+    uint32_t size = dims[i].x * dims[i].y * dims[i].z;
+    out->lo[i] = b;
+    out->hi[i] = b + size;
+    out->block_dim[i] = dims[i];
+    if (!base_line) b += size;
+  }
+  uint32_t max_thread = 0, max_block = 9999999u, total = 0;
+  for (int i = 0; i < n; i++) {
+    uint32_t size = dims[i].x * dims[i].y * dims[i].z;
+    if (size == 0) return -1;
+    if (k[i].reg != 0) {  /* the per-list tables carry no Reg; the map form requires it */
+      uint32_t mb = reg_file / k[i].reg / size;
+      if (mb < max_block) max_block = mb;
+    }
+    total += size;
+    if (size > max_thread) max_thread = size;
+  }
+  if (max_threads / total < max_block) max_block = max_threads / total;
+  out->launch_threads = base_line ? max_thread : total;
+  out->launch_blocks = launch_bound ? max_block : 0;
+  return 0;
+}
+
+/*
  * Split enumeration of the driver: tools/llvm-smart-fuser/main.cpp:215-227.
  * For a horizontal preset, Split = 128, 256, ... < d1+d2; ExecTime0 = Split,
  * ExecTime1 = (d1+d2) - Split; the variant is named "<preset>_idx_<Split/128-1>".

@@ -90,6 +90,28 @@ def context(infos, base_line=False, launch_bound=False, imbalanced=True, granule
     return out
 
 
+class PartitionN(C.Structure):
+    _fields_ = [("lo", C.c_uint32 * 4), ("hi", C.c_uint32 * 4), ("block_dim", Dim3 * 4),
+                ("launch_threads", C.c_uint32), ("launch_blocks", C.c_uint32)]
+
+
+def context_n(infos, base_line=False, launch_bound=False, imbalanced=True, granule=32,
+              reg_file=65536, max_threads=2048) -> PartitionN:
+    """infos: up to four tuples ((X,Y,Z), reg, exec_time): the Context of a list of that many kernels."""
+    n = len(infos)
+    arr = (KernelInfo * n)()
+    for i, (dim, reg, t) in enumerate(infos):
+        arr[i].block_dim = Dim3(*dim)
+        arr[i].reg = reg
+        arr[i].exec_time = t
+    out = PartitionN()
+    rc = lib().orc_context_n(arr, n, int(base_line), int(launch_bound), int(imbalanced),
+                             C.c_uint32(granule), C.c_uint32(reg_file), C.c_uint32(max_threads), C.byref(out))
+    if rc != 0:
+        raise ValueError("orc_context_n rejected the kernel table")
+    return out
+
+
 def enumerate_splits(infos, granule=32):
     arr = (KernelInfo * 2)()
     for i, (dim, reg, t) in enumerate(infos):

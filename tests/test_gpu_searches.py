@@ -267,6 +267,46 @@ def test_ethash_sia_bounded_builds(cuda, cfg):
         assert H.read_search_results(r1) == want1 and H.read_search_results(r2) == want2, waves
 
 
+def test_three_search_kernels_in_one_launch(cuda):
+    """configs/crypt_four.yaml: ccminer-Blake2b + SHA-256d + Ethash as one fused kernel (and its vertical
+    baseline), found sets of all three against the oracle."""
+    import hfuse_amd
+    t = hfuse_amd.triples_config()
+    i = t.find_fusion_n("blake2b_gpu_hash", "sha256d_gpu_hash_shared", "ethash_search")
+    n_items = 100003
+    dag = _dag(cuda, n_items, SEED)
+    header = O.seeded_bytes(32, SEED + 50)
+    hb, hs = O.seeded_bytes(80, SEED + 51), O.seeded_bytes(80, SEED + 52)
+    eth_target = (1 << 55) - 1
+    consts = H.Constants().set_ethash(dag, n_items, header, eth_target).set_sha256d(hs, EASY10).set_blake2b(hb)
+    count = 20000
+    want_b = []
+    for k in range(count):
+        nonce = (0xFFFFF000 + k) & 0xFFFFFFFF
+        d = O.ccminer_blake2b_80(hb, nonce)
+        if int.from_bytes(d[:8], "big") <= EASY10:
+            want_b.append((nonce, d, bytes(32)))
+    want_b = (len(want_b), sorted(want_b))
+    want_s = oracle_hits(O.sha256d_search(hs, 17, count, EASY10))
+    assert want_b[0] > 0 and want_s[0] > 0
+    for preset, block, grid in (("hfuse", None, 96), ("hfuse", (64, 128, 192), 64), ("hfuse_lb", None, 32), ("vfuse", None, 96)):
+        plan = t.plan(i, preset)
+        if block:
+            plan.set_block_n(*block)
+        plan.bind_constants(consts)
+        q = plan.partition_n
+        share = q.hi[2] - q.lo[2]
+        want_e = oracle_hits(O.ethash_search(None, SEED, n_items, header, 1 << 33, grid * share, eth_target))
+        assert 0 < want_e[0] <= 64
+        rb, rs, re_ = H.new_search_results(), H.new_search_results(), H.new_search_results()
+        plan.launch_n([H.blake2b_args(rb, count, 0xFFFFF000, EASY10), H.sha256d_args(rs, count, 17), H.ethash_args(re_, 1 << 33)],
+                      grid_blocks=grid)
+        sync()
+        assert H.read_search_results(rb) == want_b, preset
+        assert H.read_search_results(rs) == want_s, preset
+        assert H.read_search_results(re_) == want_e, preset
+
+
 def _strict(found_hits, limit, key):
     """The sub-set of an easy-target found set that also meets the stricter target `limit`."""
     hits = [h for h in found_hits[1] if key(h[1]) <= limit]

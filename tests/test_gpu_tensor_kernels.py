@@ -477,6 +477,62 @@ def test_bounded_builds_at_every_wave_count(cuda, cfg):
             b.check()
 
 
+def test_three_kernel_fusions(cuda):
+    """The reference's three-kernel lists (configs/im2col_maxpool_norm.yaml, maxpool_summary_norm.yaml) as one
+    fused kernel each: horizontal at the shipped block shape, other shapes, a caller's grid, the vertical
+    baseline; every output against PyTorch CPU and the oracle as for the pairs."""
+    import hfuse_amd
+    t = hfuse_amd.triples_config()
+    i = t.find_fusion_n("im2col_kernel", "MaxPoolForward", "batch_norm_collect_statistics_kernel")
+    j = t.find_fusion_n("MaxPoolForward", "kernelHistogram1D", "batch_norm_collect_statistics_kernel")
+    shapes = [(lambda: Im2col(cuda, 32, 64, 56, 56), lambda: MaxPool(cuda, 32, 64, 112, 112, (3, 3), (2, 2), (1, 1)),
+               lambda: BnStats(cuda, 32, 256, 28, 28)),
+              (lambda: Im2col(cuda, 2, 3, 9, 10), lambda: MaxPool(cuda, 2, 3, 9, 7, (2, 2), (2, 2), (0, 0)),
+               lambda: BnStats(cuda, 4, 37, 6, 5))]
+    for mk in shapes:
+        for preset, block, grid in (("hfuse", None, 0), ("hfuse", (512, 256, 256), 0), ("hfuse", (64, 64, 64), 0),
+                                    ("hfuse", (128, 192, 704), 5), ("hfuse_lb", None, 0), ("vfuse", None, 0), ("vfuse_lb", None, 3)):
+            plan = t.plan(i, preset)
+            if block:
+                plan.set_block_n(*block)
+            a, b, c = (m() for m in mk)
+            plan.launch_n([a.args, b.args, c.args], grid_blocks=grid)
+            sync()
+            a.check()
+            b.check()
+            c.check()
+    for preset, block in (("hfuse", None), ("hfuse", (256, 512, 256)), ("vfuse", None)):
+        plan = t.plan(j, preset)
+        if block:
+            plan.set_block_n(*block)
+        for n in (1 << 22, 70001):
+            a = MaxPool(cuda, 8, 32, 64, 64, (2, 2), (2, 2), (0, 0))
+            b = Histc(cuda, n)
+            c = BnStats(cuda, 8, 40, 14, 14)
+            plan.launch_n([a.args, b.args, c.args])
+            sync()
+            a.check()
+            b.check()
+            c.check()
+    # timing helper: natives back to back and the fused kernel both run the real kernels
+    plan = t.plan(i)
+    for mode in (2, 3):
+        a, b, c = (m() for m in shapes[1])
+        assert plan.time_n(mode, [[a.args, b.args, c.args]], 1, 2) > 0
+        sync()
+        a.check()
+        b.check()
+        c.check()
+    with pytest.raises(H.HfuseError):
+        plan.time_n(0, [[a.args, b.args, c.args]], 0, 1)
+    # empty work in one part
+    a, c = Im2col(cuda, 2, 3, 9, 10), BnStats(cuda, 4, 37, 6, 5)
+    b = MaxPool(cuda, 2, 3, 9, 7, (2, 2), (2, 2), (0, 0))
+    plan.launch_n([a.args, b.args, c.args], grid_blocks=1)
+    sync()
+    a.check(); b.check(); c.check()
+
+
 def test_time_pair_continues_the_rotation(cuda, cfg):
     """hf_time_pair's first_set: repetition r uses set (first_set + r) % nsets, so short calls chained
     through a Rotation touch every set.  Three sets of a tiny histogram; each launch adds its set's

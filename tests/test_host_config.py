@@ -120,7 +120,7 @@ def test_fusion_list_errors():
         Config("- File: f\n  Kernels:\n    - im2col_kernel\n    - nope\n", KERNELS_MAP)
     assert e.value.code == L.HF_EPARSE and "nope" in e.value.message
     # the schema allows any number of kernels per entry (the reference's crypt_four.yaml names three):
-    # such a list loads, and only asking for a plan of a non-pair is refused
+    # such a list loads; plans exist for entries of two and of three kernels
     cfg = Config("- File: one\n  Kernels:\n    - im2col_kernel\n"
                  "- File: three\n  Kernels:\n    - im2col_kernel\n    - MaxPoolForward\n    - im2col_kernel\n"
                  "- File: two\n  Kernels:\n    - im2col_kernel\n    - MaxPoolForward\n", KERNELS_MAP)
@@ -128,13 +128,17 @@ def test_fusion_list_errors():
     assert cfg.fusion(0) == ("one", "im2col_kernel", "")
     assert cfg.fusion_kernels(1) == ["im2col_kernel", "MaxPoolForward", "im2col_kernel"]
     assert cfg.find_fusion("im2col_kernel", "MaxPoolForward") == 2      # the triple is not mistaken for the pair
-    for i in (0, 1):
-        with pytest.raises(hfuse_amd.HfuseError) as e:
-            cfg.plan(i)
-        assert e.value.code == L.HF_EUNSUPPORTED and "pairs" in e.value.message
-        with pytest.raises(hfuse_amd.HfuseError) as e:
-            cfg.num_splits(i)
-        assert e.value.code == L.HF_EUNSUPPORTED
+    assert cfg.find_fusion_n("im2col_kernel", "MaxPoolForward", "im2col_kernel") == 1
+    with pytest.raises(hfuse_amd.HfuseError) as e:
+        cfg.plan(0)
+    assert e.value.code == L.HF_EUNSUPPORTED and "two or three" in e.value.message
+    with pytest.raises(hfuse_amd.HfuseError) as e:
+        cfg.num_splits(0)
+    assert e.value.code == L.HF_EUNSUPPORTED
+    with pytest.raises(hfuse_amd.HfuseError) as e:                      # 512 + 256 + 512 threads
+        cfg.plan(1)
+    assert e.value.code == L.HF_EINVAL and "exceeds 1024" in e.value.message
+    assert cfg.num_splits(1) == 5                                        # the loop varies the first two: 128 .. 640 < 768
     cfg.plan(2)
     with pytest.raises(hfuse_amd.HfuseError) as e:
         Config("- File: f\n  Kernels: []\n", KERNELS_MAP)
@@ -551,6 +555,135 @@ def test_launch_bound_formula_and_built_variants(cfg):
     p = cfg.plan(i, "hfuse_lb")
     p.set_launch_bound(True)
     assert p.launch_waves[1] == 8
+
+
+TRIPLE_TABLE = """
+a:
+  KernelName: im2col_kernel
+  HasBarriers: false
+  BlockDim: {bd0}
+  Reg: 42
+  ExecTime: {e0}
+b:
+  KernelName: MaxPoolForward
+  HasBarriers: false
+  BlockDim: {bd1}
+  Reg: 32
+  ExecTime: {e1}
+c:
+  KernelName: batch_norm_collect_statistics_kernel
+  HasBarriers: true
+  BlockDim: {bd2}
+  Reg: 23
+{e2}"""
+
+
+def _triple_cfg(dims, times):
+    def bd(d):
+        return "\n    X: %d\n    Y: %d\n    Z: 1" % d
+    e2 = "  ExecTime: %s\n" % times[2] if times[2] is not None else ""
+    return Config("- File: t\n  Kernels:\n    - a\n    - b\n    - c\n",
+                  TRIPLE_TABLE.format(bd0=bd(dims[0]), bd1=bd(dims[1]), bd2=bd(dims[2]), e0=times[0], e1=times[1], e2=e2))
+
+
+def test_three_kernel_partition_matches_oracle():
+    """Plans of three-kernel entries against the oracle's Context of three (64-lane granule, this part's
+    register file): table split, every index of the driver's split loop, the ExecTime split, the vertical
+    presets, the launch-bound hint, the local index remap; refusals are parts that are empty, ragged or do
+    not divide by BlockDim.Y, and blocks beyond 1024 threads."""
+    import random
+    rng = random.Random(31337)
+    regs = (42, 32, 23)
+    checked = refused = 0
+    for case in range(120):
+        dims = []
+        for y in (1, 1, rng.choice([1, 4, 8])):
+            t = rng.choice([64, 128, 192, 256, 320, 512])
+            dims.append((t // y, y))
+        times = [rng.choice([5.0, 17.0, 31.0, 95.0]) for _ in range(3)]
+        no_e2 = rng.random() < 0.3
+        cfg = _triple_cfg(dims, times[:2] + [None if no_e2 else times[2]])
+        total = sum(x * y for x, y in dims)
+        d01 = dims[0][0] * dims[0][1] + dims[1][0] * dims[1][1]
+
+        def rows(e):
+            return [((dims[i][0], dims[i][1], 1), regs[i], e[i]) for i in range(3)]
+        variants = [(L.HF_SPLIT_TABLE, rows(times), False)]
+        for idx in range(cfg.num_splits(0)):
+            variants.append((idx, rows([128.0 * (idx + 1), d01 - 128.0 * (idx + 1), -1.0 if no_e2 else times[2]]), True))
+        assert cfg.num_splits(0) == len(range(128, d01, 128))
+        if not no_e2:
+            variants.append((L.HF_SPLIT_EXECTIME, rows(times), True))
+        for idx, ex, imb in variants:
+            for preset, lb in (("hfuse", False), ("hfuse_lb", True)):
+                try:
+                    want = O.context_n(ex, launch_bound=lb, imbalanced=imb, granule=64, reg_file=4 * 512 * 64, max_threads=2048)
+                except ValueError:
+                    want = None
+                try:
+                    plan = cfg.plan(0, preset, idx)
+                except hfuse_amd.HfuseError as e:
+                    assert e.code == L.HF_EINVAL
+                    refused += 1
+                    if want is not None:
+                        parts = [want.hi[h] - want.lo[h] for h in range(3)]
+                        assert sum(parts) > 1024 or any(p == 0 or p > 1 << 20 or p % 64 or p % dims[h][1] for h, p in enumerate(parts)), (dims, idx, parts)
+                    continue
+                got = plan.partition_n
+                assert want is not None and got.n == 3 and plan.num_kernels == 3
+                assert list(got.lo)[:3] == list(want.lo)[:3] and list(got.hi)[:3] == list(want.hi)[:3], (dims, idx)
+                for h in range(3):
+                    assert (got.block_dim[h].x, got.block_dim[h].y) == (want.block_dim[h].x, want.block_dim[h].y)
+                    tid = rng.randrange(got.lo[h], got.hi[h])
+                    assert plan.local_index(h, tid) == O.remap_tid(tid, got.lo[h], (got.block_dim[h].x, got.block_dim[h].y, 1))
+                assert got.launch_threads == want.launch_threads and got.launch_blocks == want.launch_blocks
+                checked += 1
+        for preset, lb in (("vfuse", False), ("vfuse_lb", True)):
+            want = O.context_n(rows(times), base_line=True, launch_bound=lb, imbalanced=False, granule=64,
+                               reg_file=4 * 512 * 64, max_threads=2048)
+            got = cfg.plan(0, preset, 0).partition_n
+            assert list(got.lo)[:3] == [0, 0, 0] and list(got.hi)[:3] == list(want.hi)[:3]
+            assert got.launch_threads == want.launch_threads and got.launch_blocks == want.launch_blocks
+            checked += 1
+    assert checked > 300 and refused > 20
+
+
+def test_three_kernel_plans_refuse_the_calls_that_shape_a_pair():
+    cfg = _triple_cfg([(256, 1), (256, 1), (32, 8)], [1.0, 1.0, 1.0])
+    plan = cfg.plan(0)
+    lib = L.lib()
+    assert plan.partition_n.name.decode() == "im2col_kernel_MaxPoolForward_batch_norm_collect_statistics_kernel_fused_kernel_hfuse_table"
+    for call in (lambda: plan.set_block(128, 128), lambda: plan.set_grids(1, 1), lambda: plan.set_lending(True),
+                 lambda: plan.set_barrier_mode(L.HF_BARRIER_BLOCKIDX), lambda: plan.set_launch_bound(True),
+                 lambda: plan.set_launch_waves(8), lambda: plan.partition, lambda: plan.local_index(3, 0)):
+        with pytest.raises(hfuse_amd.HfuseError) as e:
+            call()
+        assert e.value.code == L.HF_EINVAL
+    a = L.Im2colArgs()
+    assert lib.hf_launch_fused(plan._h, C.byref(a), C.byref(a), 0, None) == L.HF_EINVAL
+    ptrs = (C.c_void_p * 3)(C.addressof(a), C.addressof(a), C.addressof(a))
+    assert lib.hf_launch_fused_n(plan._h, ptrs, 2, 0, None) == L.HF_EINVAL         # three lists for three kernels
+    assert lib.hf_launch_fused_n(plan._h, ptrs, 3, 0, None) == L.HF_EINVAL         # null data pointers: refused on the host
+    assert b"null data pointer" in lib.hf_last_error()
+    with pytest.raises(hfuse_amd.HfuseError):
+        cfg.plan(0, "hfuse", L.HF_SPLIT_TABLE, 128)                                 # split_threads shapes a pair
+    plan.set_block_n(128, 512, 256)
+    q = plan.partition_n
+    assert list(q.hi)[:3] == [128, 640, 896] and q.name.decode().endswith("_hfuse_block_128_512_256")
+    assert (q.block_dim[2].x, q.block_dim[2].y) == (32, 8)
+    for bad in ((128, 512), (128, 512, 100), (512, 512, 512), (64, 64, 68), (0, 64, 64)):
+        with pytest.raises(hfuse_amd.HfuseError):
+            plan.set_block_n(*bad)
+    # a pair through the n-kernel calls
+    pair = Config(FUSION, KERNELS_MAP).plan(0)
+    pair.set_block_n(128, 256)
+    assert list(pair.partition_n.hi)[:2] == [128, 384] and pair.partition_n.n == 2
+    # the shipped three-kernel list and its Blocks key
+    t = hfuse_amd.triples_config()
+    assert [list(t.plan(i).partition_n.hi)[:3] for i in range(3)] == [[128, 256, 384], [256, 640, 768], [128, 768, 896]]
+    with pytest.raises(hfuse_amd.HfuseError) as e:
+        Config("- File: t\n  Kernels:\n    - a\n    - b\n  Blocks:\n    - 64\n    - 64\n", KERNELS_MAP.replace("im2col_kernel:", "a:").replace("MaxPoolForward:", "b:"))
+    assert e.value.code == L.HF_EPARSE and "Blocks" in e.value.message
 
 
 def test_header_symbols_are_all_exported():

@@ -70,3 +70,31 @@ def test_remap_is_the_documented_formula_and_a_bijection():
         n = dim[0] * dim[1] * dim[2]
         seen = {O.remap_tid(lo + t, lo, dim) for t in range(n)}
         assert seen == set(itertools.product(range(dim[0]), range(dim[1]), range(dim[2])))
+
+
+def test_context_of_three_kernels_hand_worked():
+    """orc_context_n against numbers worked by hand through include/KernelFusion.h:45-80 and
+    lib/KernelFuser/KernelPrinter.cpp:46-66 (32-thread granule, 64 K registers, 2048 threads, as the reference)."""
+    # configs/im2col_maxpool_norm.yaml: 512x1, 256x1, 32x8 -- plain concatenation
+    rows = [((512, 1, 1), 32, -1.0), ((256, 1, 1), 32, -1.0), ((32, 8, 1), 32, -1.0)]
+    p = O.context_n(rows, imbalanced=False, launch_bound=True)
+    assert list(p.lo)[:3] == [0, 512, 768] and list(p.hi)[:3] == [512, 768, 1024]
+    assert p.launch_threads == 1024
+    # min(65536/32/512 = 4, 65536/32/256 = 8, 8, 2048/1024 = 2) = 2
+    assert p.launch_blocks == 2
+    v = O.context_n(rows, base_line=True, imbalanced=False)
+    assert list(v.lo)[:3] == [0, 0, 0] and list(v.hi)[:3] == [512, 256, 256] and v.launch_threads == 512 and v.launch_blocks == 0
+    # ExecTimes 1 : 2 : 1 over 1024 threads: int(0.25 * 1024 / 32) * 32 = 256, int(0.5 * 32) * 32 = 512, rest 256
+    timed = [((512, 1, 1), 32, 10.0), ((256, 1, 1), 32, 20.0), ((32, 8, 1), 32, 10.0)]
+    q = O.context_n(timed, imbalanced=True)
+    assert [q.hi[i] - q.lo[i] for i in range(3)] == [256, 512, 256]
+    assert (q.block_dim[2].x, q.block_dim[2].y) == (32, 8) and q.block_dim[1].x == 512
+    # the driver's split loop on three kernels (main.cpp:219-225): Split 128 of 768 for the first two, the third
+    # keeps ExecTime -1: total time 767; int(128/767 * 32) = 5 -> 160, int(640/767 * 32) = 26 -> 832, rest 1024 - 992 = 32
+    loop = [((512, 1, 1), 32, 128.0), ((256, 1, 1), 32, 640.0), ((32, 8, 1), 32, -1.0)]
+    r = O.context_n(loop, imbalanced=True)
+    assert [r.hi[i] - r.lo[i] for i in range(3)] == [160, 832, 32]
+    # a pair through the n-kernel routine equals the two-kernel routine
+    pair = [((512, 1, 1), 49, 31.0), ((256, 1, 1), 24, 95.0)]
+    a, b = O.context_n(pair, launch_bound=True), O.context(pair, launch_bound=True)
+    assert list(a.hi)[:2] == list(b.hi) and a.launch_blocks == b.launch_blocks and a.launch_threads == b.launch_threads

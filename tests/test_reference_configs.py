@@ -48,13 +48,24 @@ def test_per_pair_tables():
     assert seen == 16
 
 
-def test_lists_of_three_kernels_load_and_are_refused_as_plans():
+def test_lists_of_three_kernels_load_and_plan():
+    """The reference's three-kernel lists: the Context's partition among three at the table's block shapes."""
+    want = {"crypt_four.yaml": [128, 256, 384], "im2col_maxpool_norm.yaml": [512, 768, 1024]}
     for name, n in MANY.items():
         cfg = Config.from_files(None, os.path.join(REF, name))
         assert cfg.num_fusions == 1 and len(cfg.fusion_kernels(0)) == n
-        with pytest.raises(hfuse_amd.HfuseError) as e:
-            cfg.plan(0)
-        assert e.value.code == L.HF_EUNSUPPORTED
+        if n != 3:
+            continue
+        v = cfg.plan(0, "vfuse").partition_n
+        assert v.n == 3 and list(v.lo)[:3] == [0, 0, 0]
+        if name in want:
+            part = cfg.plan(0).partition_n
+            assert list(part.hi)[:3] == want[name] and part.launch_threads == want[name][2]
+            assert part.name.decode() == "_".join(cfg.fusion_kernels(0)) + "_fused_kernel_hfuse_table"
+        else:   # maxpool_summary_norm.yaml: 256 + 512 + 512 threads do not fit one workgroup
+            with pytest.raises(hfuse_amd.HfuseError) as e:
+                cfg.plan(0)
+            assert e.value.code == L.HF_EINVAL and "exceeds 1024" in e.value.message
 
 
 def test_the_toy_file_names_kernels_this_library_does_not_have():
