@@ -71,6 +71,9 @@ def parse():
     ap.add_argument("--search-log2", type=int, default=None, help="override log2 of the nonce ranges (profiling runs)")
     ap.add_argument("--extra-pairs", action="store_true",
                     help="also time the other tensor pairs of the shipped fusion list (the reference's ml_fusion.yaml)")
+    ap.add_argument("--triples", action="store_true",
+                    help="also time the three-kernel fusions of the reference's lists (im2col + max_pool2d + bn-stats at "
+                         "the benchmark shapes; ccminer-Blake2b + SHA-256d + Ethash at 2^26 + 2^26 + 2^24 nonces)")
     ap.add_argument("--read-footprint-mb", type=int, default=0,
                     help="MB the smaller read stream of a tensor pair cycles through before a buffer set repeats "
                          "(default 600; below about 300 the memory-side cache serves the reads; at least three sets in any case)")
@@ -337,6 +340,66 @@ def run_search_pair(cfg, name, log2_a, log2_b, sweep, fused_only, steps=0, warmu
     return res
 
 
+# ------------------------------------------------------------------ three-kernel fusions
+def time_triples(rotations):
+    """The reference's three-kernel lists: the three native kernels back to back against the fused and the vertical kernel."""
+    import torch
+    import hfuse_amd
+    from hfuse_amd import launcher as H
+    from hfuse_amd import workloads as W
+    t = hfuse_amd.triples_config()
+    out = {}
+    # im2col + max_pool2d + bn-stats at the benchmark shapes, rotating buffer sets
+    names = ("im2col_kernel", "MaxPoolForward", "batch_norm_collect_statistics_kernel")
+    makers = [W.kernel_workload(k) for k in names]
+    sets, read = [], 0
+    while read < W.MIN_READ_FOOTPRINT:
+        made = [mk(len(sets)) for mk, _ in makers]
+        sets.append(made)
+        read += min(m["read_bytes"] for m in made)
+    arg_sets = [[m["args"] for m in made] for made in sets]
+    nbytes = sum(b for _, b in makers)
+    i = t.find_fusion_n(*names)
+    rot = H.Rotation()
+    per = max(1, rotations) * len(sets)
+    runs = [("t_b2b_ms", t.plan(i), 2), ("t_fused_ms", t.plan(i), 3), ("t_vfuse_ms", t.plan(i, "vfuse"), 3)]
+    for _, p, m in runs:
+        p.time_n(m, arg_sets, 0, len(sets), rotation=rot)
+    samples = {k: [] for k, _, _ in runs}
+    for _ in range(5):
+        for key, p, m in runs:
+            samples[key].append(p.time_n(m, arg_sets, 2, per, rotation=rot) / per)
+    r = {k: statistics.median(v) for k, v in samples.items()}
+    r["speedup_pct"] = (r["t_b2b_ms"] / r["t_fused_ms"] - 1.0) * 100.0
+    r["fused_gbps"] = nbytes / (r["t_fused_ms"] * 1e-3) / 1e9
+    r["threads"] = [int(x) for x in list(t.plan(i).partition_n.hi)[:3]]
+    r["buffer_sets"] = len(sets)
+    out["im2col+max_pool2d+bn_stats"] = r
+    del sets, arg_sets
+    torch.cuda.empty_cache()
+    # ccminer-Blake2b + SHA-256d + Ethash (4 GiB DAG)
+    la, lb, le = 26, 26, 24
+    sp = W.SearchPair("ethash_search", "sha256d_gpu_hash_shared", le, lb)    # uploads the DAG and two headers
+    sp.constants.set_blake2b(W.splitmix64_bytes(80, SEED + 102))
+    j = t.find_fusion_n("blake2b_gpu_hash", "sha256d_gpu_hash_shared", "ethash_search")
+    rb, rs, re_ = H.new_search_results(), H.new_search_results(), H.new_search_results()
+    args = [[H.blake2b_args(rb, 1 << la, 0, W.SearchPair.TARGET32), H.sha256d_args(rs, 1 << lb, 0), H.ethash_args(re_, 0)]]
+    res = {}
+    for key, preset, mode in (("t_b2b_ms", "hfuse", 2), ("t_fused_ms", "hfuse", 3), ("t_vfuse_ms", "vfuse", 3)):
+        plan = t.plan(j, preset)
+        plan.bind_constants(sp.constants)
+        q = plan.partition_n
+        share = 128 if mode == 2 else q.hi[2] - q.lo[2]      # Ethash scans grid * its threads nonces
+        grid = (1 << le) // share
+        res[key] = statistics.median([plan.time_n(mode, args, 0, 1, grid) for _ in range(3)])
+    res["speedup_pct"] = (res["t_b2b_ms"] / res["t_fused_ms"] - 1.0) * 100.0
+    res["log2_nonces"] = [la, lb, le]
+    out["blake2b+sha256d+ethash"] = res
+    del sp
+    torch.cuda.empty_cache()
+    return out
+
+
 # ------------------------------------------------------------------ CPU baseline
 def cpu_baseline_tensor(name, budget_s=8.0):
     """PyTorch's CPU operators (the reference CPU path) and the C restatement (OpenMP) on the full shape of
@@ -522,6 +585,8 @@ def main():
                 del pair
                 torch.cuda.empty_cache()
 
+    triples = time_triples(args.rotations) if args.triples else None
+
     cpu = None
     found = {n: report[n].pop("_found") for n in names if n in SEARCH_NAMES}
     if not args.no_cpu:
@@ -604,6 +669,8 @@ def main():
     }
     if extra:
         line["extra_pairs"] = extra
+    if triples:
+        line["three_kernel_fusions"] = triples
     print(json.dumps(line))
 
 
