@@ -769,22 +769,9 @@ struct HistcBody {
       if (sb.bid == 0 && (int64_t)sb.tid < head) count<POW2, GLOBAL>(bins, b[sb.tid], lo, hi, fn, range, inv_range, inv_lo, inv_hi, nbins);
       b += head;
       const int64_t rest = total - head;
-#ifndef HF_HIST_CONTIG
-#define HF_HIST_CONTIG 0
-#endif
-#if HF_HIST_CONTIG
-      // every workgroup walks one contiguous run of the input (a whole number of block-wide rows)
-      const int64_t nall = rest >> 2;
-      const int64_t rows = (nall + sb.nthreads - 1) / sb.nthreads;
-      const int64_t per = (rows + sb.nblocks - 1) / sb.nblocks * sb.nthreads;
-      const int64_t n4 = min(nall, (int64_t)(sb.bid + 1) * per);
-      const int64_t stride = (int64_t)sb.nthreads;
-      int64_t i = (int64_t)sb.bid * per + sb.tid;
-#else
       const int64_t n4 = rest >> 2;
       const int64_t stride = (int64_t)sb.gstride();
       int64_t i = (int64_t)sb.gtid();
-#endif
       // Several 16-byte loads in flight per lane before the dependent LDS atomics: eight with up to
       // eight wavefronts, four with more (about 48-64 KB in flight per CU either way; beyond that the
       // memory system gets slower, and more wavefronts with shorter batches overlap their arithmetic better).

@@ -111,28 +111,11 @@ struct FuseGeom {
 
 constexpr unsigned kBarrierWords = 4;  // 16 bytes reserved at the base of LDS for arrival counters
 
-// Workgroups are dealt to the eight XCDs round-robin by their index.  This renumbering gives the
-// workgroups of one XCD consecutive virtual indices: XCD x owns the x-th contiguous eighth of the
-// index range (the first grid % 8 XCDs hold one workgroup more).
-constexpr unsigned kXcds = 8;
-__device__ __forceinline__ unsigned xcd_contiguous(unsigned bid, unsigned grid) {
-  const unsigned xcd = bid % kXcds, slot = bid / kXcds;
-  const unsigned q = grid / kXcds, r = grid % kXcds;
-  return xcd * q + (xcd < r ? xcd : r) + slot;
-}
-
 // Native launch: the body owns the whole workgroup.
 template <class K, int T>
 __global__ __launch_bounds__(T) void native_kernel(typename K::Args a, unsigned hint) {
   extern __shared__ __align__(16) unsigned char smem[];
-#ifndef HF_XCD_SWIZZLE
-#define HF_XCD_SWIZZLE 0
-#endif
-#if HF_XCD_SWIZZLE
-  const unsigned bid = xcd_contiguous(blockIdx.x, gridDim.x);
-#else
   const unsigned bid = blockIdx.x;
-#endif
   SubBlock<BAR_WORKGROUP> sb{threadIdx.x, blockDim.x, bid, gridDim.x, nullptr, 0,
                              bid * blockDim.x, gridDim.x * blockDim.x};
   K::run(a, sb, smem, hint);
