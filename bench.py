@@ -351,51 +351,38 @@ def time_triples(rotations):
     out = {}
     # im2col + max_pool2d + bn-stats at the benchmark shapes, rotating buffer sets
     names = ("im2col_kernel", "MaxPoolForward", "batch_norm_collect_statistics_kernel")
-    makers = [W.kernel_workload(k) for k in names]
-    sets, read = [], 0
-    while read < W.MIN_READ_FOOTPRINT:
-        made = [mk(len(sets)) for mk, _ in makers]
-        sets.append(made)
-        read += min(m["read_bytes"] for m in made)
-    arg_sets = [[m["args"] for m in made] for made in sets]
-    nbytes = sum(b for _, b in makers)
+    work = W.TensorTriple(names)
     i = t.find_fusion_n(*names)
-    rot = H.Rotation()
-    per = max(1, rotations) * len(sets)
+    nsets = len(work.sets)
+    per = max(1, rotations) * nsets
     runs = [("t_b2b_ms", t.plan(i), 2), ("t_fused_ms", t.plan(i), 3), ("t_vfuse_ms", t.plan(i, "vfuse"), 3)]
     for _, p, m in runs:
-        p.time_n(m, arg_sets, 0, len(sets), rotation=rot)
+        work.time(p, m, 0, nsets)
     samples = {k: [] for k, _, _ in runs}
     for _ in range(5):
         for key, p, m in runs:
-            samples[key].append(p.time_n(m, arg_sets, 2, per, rotation=rot) / per)
+            samples[key].append(work.time(p, m, 2, per) / per)
     r = {k: statistics.median(v) for k, v in samples.items()}
     r["speedup_pct"] = (r["t_b2b_ms"] / r["t_fused_ms"] - 1.0) * 100.0
-    r["fused_gbps"] = nbytes / (r["t_fused_ms"] * 1e-3) / 1e9
+    r["fused_gbps"] = work.bytes / (r["t_fused_ms"] * 1e-3) / 1e9
     r["threads"] = [int(x) for x in list(t.plan(i).partition_n.hi)[:3]]
-    r["buffer_sets"] = len(sets)
+    r["buffer_sets"] = nsets
     out["im2col+max_pool2d+bn_stats"] = r
-    del sets, arg_sets
+    del work
     torch.cuda.empty_cache()
     # ccminer-Blake2b + SHA-256d + Ethash (4 GiB DAG)
-    la, lb, le = 26, 26, 24
-    sp = W.SearchPair("ethash_search", "sha256d_gpu_hash_shared", le, lb)    # uploads the DAG and two headers
-    sp.constants.set_blake2b(W.splitmix64_bytes(80, SEED + 102))
-    j = t.find_fusion_n("blake2b_gpu_hash", "sha256d_gpu_hash_shared", "ethash_search")
-    rb, rs, re_ = H.new_search_results(), H.new_search_results(), H.new_search_results()
-    args = [[H.blake2b_args(rb, 1 << la, 0, W.SearchPair.TARGET32), H.sha256d_args(rs, 1 << lb, 0), H.ethash_args(re_, 0)]]
+    st = W.SearchTriple((26, 26, 24))
+    j = t.find_fusion_n(*W.SearchTriple.KERNELS)
     res = {}
     for key, preset, mode in (("t_b2b_ms", "hfuse", 2), ("t_fused_ms", "hfuse", 3), ("t_vfuse_ms", "vfuse", 3)):
         plan = t.plan(j, preset)
-        plan.bind_constants(sp.constants)
-        q = plan.partition_n
-        share = 128 if mode == 2 else q.hi[2] - q.lo[2]      # Ethash scans grid * its threads nonces
-        grid = (1 << le) // share
-        res[key] = statistics.median([plan.time_n(mode, args, 0, 1, grid) for _ in range(3)])
+        res[key] = statistics.median([st.time(plan, mode) for _ in range(3)])
     res["speedup_pct"] = (res["t_b2b_ms"] / res["t_fused_ms"] - 1.0) * 100.0
-    res["log2_nonces"] = [la, lb, le]
+    res["vfuse_speedup_pct"] = (res["t_b2b_ms"] / res["t_vfuse_ms"] - 1.0) * 100.0
+    res["threads"] = [int(x) for x in list(t.plan(j).partition_n.hi)[:3]]
+    res["log2_nonces"] = list(st.log2)
     out["blake2b+sha256d+ethash"] = res
-    del sp
+    del st
     torch.cuda.empty_cache()
     return out
 

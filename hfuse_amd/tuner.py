@@ -188,6 +188,112 @@ def tune(cfg: H.Config, fusion_index: int, args1: Sequence, args2: Sequence, *,
                             [(final[i][1].label(), t) for t, i in med if final[i][1].bounded])
 
 
+# ------------------------------------------------------------------ three-kernel entries
+def triple_block_candidates(cfg: H.Config, fusion_index: int, max_block: int, step: int = WAVE) -> List[Tuple[int, int, int]]:
+    """Every (threads0, threads1, threads2) a three-kernel entry can run with: positive multiples of `step`
+    that divide by each kernel's BlockDim.Y, total <= max_block."""
+    ys = [cfg.kernel(k).block_dim.y for k in cfg.fusion_kernels(fusion_index)]
+    out = []
+    for t0 in range(step, max_block, step):
+        for t1 in range(step, max_block - t0, step):
+            for t2 in range(step, max_block - t0 - t1 + 1, step):
+                if t0 % ys[0] == 0 and t1 % ys[1] == 0 and t2 % ys[2] == 0:
+                    out.append((t0, t1, t2))
+    return out
+
+
+def tune_triple(cfg: H.Config, fusion_index: int, time_fused, blocks: Sequence[Tuple[int, int, int]], *,
+                finalists: int = 4, verbose: bool = False):
+    """Sweep the block shapes of a three-kernel entry.  `time_fused(plan)` returns milliseconds per launch of
+    the plan on the caller's workload.  -> (best shape, its time, [(shape, ms), ...] of the whole sweep); the
+    `finalists` fastest are timed three more times and the median decides."""
+    probed = []
+    for shape in blocks:
+        plan = cfg.plan(fusion_index)
+        try:
+            plan.set_block_n(*shape)
+        except H.HfuseError:
+            continue
+        t = time_fused(plan)
+        probed.append((t, shape, plan))
+        if verbose:
+            print(f"  {'+'.join(map(str, shape)):16s} {t * 1e3:9.2f} us", file=sys.stderr, flush=True)
+    if not probed:
+        raise RuntimeError("no legal block shape")
+    probed.sort(key=lambda r: r[0])
+    final = probed[:max(1, finalists)]
+    med = sorted((statistics.median([time_fused(plan) for _ in range(3)]), shape) for _, shape, plan in final)
+    return med[0][1], med[0][0], [(shape, t) for t, shape, _ in probed]
+
+
+def apply_blocks_to_fusion_yaml(text: str, shapes: dict) -> str:
+    """Return the fusion list `text` with `Blocks:` of the entries in `shapes` {entry index: (t0, t1, t2)}
+    replaced (or added); every other line is kept."""
+    lines = text.splitlines()
+    starts = [i for i, ln in enumerate(lines) if ln.startswith("- ")] + [len(lines)]
+    out: List[str] = lines[:starts[0]] if starts else list(lines)
+    for n in range(len(starts) - 1):
+        entry = lines[starts[n]:starts[n + 1]]
+        if n in shapes:
+            kept, skipping = [], False
+            for ln in entry:
+                if re.match(r"^\s+Blocks\s*:", ln):
+                    skipping = True
+                    continue
+                if skipping and re.match(r"^\s+-\s+\d+\s*$", ln):
+                    continue
+                skipping = False
+                kept.append(ln)
+            tail = []
+            while kept and (not kept[-1].strip() or kept[-1].lstrip().startswith("#")):
+                tail.insert(0, kept.pop())
+            kept.append("  Blocks:")
+            kept.extend(f"    - {t}" for t in shapes[n])
+            entry = kept + tail
+        out.extend(entry)
+    return "\n".join(out) + "\n"
+
+
+def tune_shipped_triples(out_path: str, verbose: bool = False, search_log2=(26, 26, 24)) -> int:
+    """Tune the block shapes of the shipped three-kernel list on the benchmark workloads and write it to `out_path`."""
+    import torch
+    from . import workloads as W
+    here = os.path.join(os.path.dirname(os.path.abspath(__file__)), "configs")
+    path = os.path.join(here, "gfx950_triples.yaml")
+    text = open(path).read()
+    cfg = H.Config(text, open(os.path.join(here, "gfx950_kernels.yaml")).read())
+    shapes = {}
+    for i in range(cfg.num_fusions):
+        names = cfg.fusion_kernels(i)
+        if len(names) != 3:
+            continue
+        print(f"[{i}] {' + '.join(names)}", file=sys.stderr, flush=True)
+        if all(k in W.TENSOR_KERNELS for k in names):
+            work = W.TensorTriple(names)
+            n = len(work.sets)
+            time_fused = lambda plan: work.time(plan, 3, 2, n) / n
+            blocks = triple_block_candidates(cfg, i, MAX_TENSOR_BLOCK, 2 * WAVE)
+            base = cfg.plan(i, "vfuse")
+            t_b2b = statistics.median([work.time(base, 2, 2, n) / n for _ in range(3)])
+        elif tuple(names) == W.SearchTriple.KERNELS:
+            work = W.SearchTriple(search_log2)
+            time_fused = lambda plan: work.time(plan, 3)
+            blocks = triple_block_candidates(cfg, i, MAX_SEARCH_BLOCK, WAVE)
+            t_b2b = statistics.median([work.time(cfg.plan(i, "vfuse"), 2) for _ in range(3)])
+        else:
+            continue
+        best, t_best, table = tune_triple(cfg, i, time_fused, blocks, verbose=verbose)
+        shapes[i] = best
+        print(f"    best {'+'.join(map(str, best))}: {t_best * 1e3:.2f} us, three natives back to back {t_b2b * 1e3:.2f} us "
+              f"({(t_b2b / t_best - 1) * 100:+.1f} %)", file=sys.stderr, flush=True)
+        del work
+        torch.cuda.empty_cache()
+    with open(out_path, "w") as f:
+        f.write(apply_blocks_to_fusion_yaml(text, shapes))
+    print(f"wrote {out_path} ({len(shapes)} entries tuned)", file=sys.stderr)
+    return 0
+
+
 # ------------------------------------------------------------------ fusion list rewriting
 _TUNED_KEY = re.compile(r"^\s+(Split|Threads|Lending|Barrier|LaunchBound)\s*:")
 BARRIER_NAMES = {L.HF_BARRIER_NONE: "none", L.HF_BARRIER_MATCHED: "matched", L.HF_BARRIER_SUBSET: "subset",
@@ -254,7 +360,11 @@ def main(argv=None) -> int:
                     help="also try the block-index partition (each workgroup runs one of the two kernels), "
                          "written as 'Barrier: blockidx' where it wins")
     ap.add_argument("--verbose", action="store_true")
+    ap.add_argument("--triples", action="store_true",
+                    help="tune the block shapes (`Blocks:`) of the shipped three-kernel list instead of the pairs")
     args = ap.parse_args(argv)
+    if args.triples:
+        return tune_shipped_triples(args.out, args.verbose)
 
     import torch
     from . import workloads as W

@@ -213,3 +213,53 @@ class SearchPair:
         from . import launcher as H
         r1, r2 = H.new_search_results(), H.new_search_results()
         return r1, r2, self._args(self.k1, r1, self.nonces[0]), self._args(self.k2, r2, self.nonces[1])
+
+
+class TensorTriple:
+    """Three tensor kernels at their benchmark shapes with rotating buffer sets: `arg_sets[s][k]`."""
+
+    def __init__(self, names, min_read_footprint=None):
+        from .launcher import Rotation
+        if min_read_footprint is None:
+            min_read_footprint = MIN_READ_FOOTPRINT
+        makers = [kernel_workload(k) for k in names]
+        self.names = tuple(names)
+        self.bytes = sum(b for _, b in makers)
+        self.sets, read = [], 0
+        while read < min_read_footprint or len(self.sets) < 3:
+            made = [mk(len(self.sets)) for mk, _ in makers]
+            self.sets.append(made)
+            read += min(m["read_bytes"] for m in made)
+        self.arg_sets = [[m["args"] for m in made] for made in self.sets]
+        self.rotation = Rotation()
+
+    def time(self, plan, mode, warmup, iters, grid_blocks=0):
+        """Milliseconds of `iters` repetitions (mode 2: the three natives back to back, 3: the fused kernel)."""
+        return plan.time_n(mode, self.arg_sets, warmup, iters, grid_blocks, rotation=self.rotation)
+
+
+class SearchTriple:
+    """ccminer-Blake2b + SHA-256d + Ethash (the reference's configs/crypt_four.yaml) over seeded headers and
+    the seeded 4 GiB DAG: 2^log2[0] + 2^log2[1] + 2^log2[2] nonces.  Bind `constants` to the plan."""
+
+    KERNELS = ("blake2b_gpu_hash", "sha256d_gpu_hash_shared", "ethash_search")
+
+    def __init__(self, log2=(26, 26, 24), dag_items=SearchPair.ETHASH_ITEMS):
+        from . import launcher as H
+        self.log2 = tuple(log2)
+        self._pair = SearchPair("ethash_search", "sha256d_gpu_hash_shared", log2[2], log2[1], dag_items)
+        self.constants = self._pair.constants
+        self.constants.set_blake2b(splitmix64_bytes(80, SEED + 102))
+        self._results = [H.new_search_results() for _ in range(3)]
+        self.args = [H.blake2b_args(self._results[0], 1 << log2[0], 0, SearchPair.TARGET32),
+                     H.sha256d_args(self._results[1], 1 << log2[1], 0), H.ethash_args(self._results[2], 0)]
+
+    def grid(self, ethash_threads: int) -> int:
+        """Workgroups that make Ethash scan its 2^log2[2] nonces with `ethash_threads` threads a block."""
+        return (1 << self.log2[2]) // ethash_threads
+
+    def time(self, plan, mode, iters=1):
+        plan.bind_constants(self.constants)
+        q = plan.partition_n
+        share = 128 if mode == 2 else q.hi[2] - q.lo[2]   # the native Ethash launch runs 128-thread blocks
+        return plan.time_n(mode, [self.args], 0, iters, self.grid(share)) / iters

@@ -680,7 +680,7 @@ def test_three_kernel_plans_refuse_the_calls_that_shape_a_pair():
     assert list(pair.partition_n.hi)[:2] == [128, 384] and pair.partition_n.n == 2
     # the shipped three-kernel list and its Blocks key
     t = hfuse_amd.triples_config()
-    assert [list(t.plan(i).partition_n.hi)[:3] for i in range(3)] == [[128, 256, 384], [256, 640, 768], [128, 768, 896]]
+    assert [list(t.plan(i).partition_n.hi)[:3] for i in range(3)] == [[64, 192, 256], [256, 640, 768], [512, 768, 1024]]
     with pytest.raises(hfuse_amd.HfuseError) as e:
         Config("- File: t\n  Kernels:\n    - a\n    - b\n  Blocks:\n    - 64\n    - 64\n", KERNELS_MAP.replace("im2col_kernel:", "a:").replace("MaxPoolForward:", "b:"))
     assert e.value.code == L.HF_EPARSE and "Blocks" in e.value.message
