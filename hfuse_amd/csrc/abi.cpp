@@ -742,6 +742,10 @@ HF_API int hf_plan_create(const hf_config *cfg, int fusion_index, const char *pr
       delete plan;
       return fail(HF_EINVAL, "split_threads shapes a pair; give a three-kernel plan its block with hf_plan_set_block_n");
     }
+    if (f.split || f.threads || f.lending >= 0 || f.barrier >= 0 || f.launch_bound >= 0) {
+      delete plan;
+      return fail(HF_EINVAL, "fusion '" + f.file + "': Split / Threads / Lending / Barrier / LaunchBound shape a pair; a three-kernel entry takes 'Blocks'");
+    }
     // the entry's own block shape (`Blocks:`), applied like a pair's Split / Threads: to the table split of a horizontal preset
     KernelRow shaped[kMaxFuse] = {plan->rows[0], plan->rows[1], plan->rows[2]};
     const bool own_shape = split_idx == HF_SPLIT_TABLE && f.blocks.size() == 3 && !p->base_line;

@@ -674,6 +674,12 @@ def test_three_kernel_plans_refuse_the_calls_that_shape_a_pair():
     for bad in ((128, 512), (128, 512, 100), (512, 512, 512), (64, 64, 68), (0, 64, 64)):
         with pytest.raises(hfuse_amd.HfuseError):
             plan.set_block_n(*bad)
+    # the keys that tune a pair do not apply to a three-kernel entry
+    keyed = Config("- File: t\n  Kernels:\n    - im2col_kernel\n    - MaxPoolForward\n    - batch_norm_collect_statistics_kernel\n  Split: 128\n",
+                   KERNELS_MAP.replace("X: 512", "X: 256", 1))
+    with pytest.raises(hfuse_amd.HfuseError) as e:
+        keyed.plan(0)
+    assert e.value.code == L.HF_EINVAL and "Blocks" in e.value.message
     # a pair through the n-kernel calls
     pair = Config(FUSION, KERNELS_MAP).plan(0)
     pair.set_block_n(128, 256)
