@@ -8,7 +8,8 @@
  * the same enumeration through the C-ABI and prints one line per variant: the fused
  * kernel's name, each kernel's thread bounds and block shape, the launch block and
  * the launch-bounds hint -- the numbers a caller needs to launch the variant with
- * hf_plan_create + hf_launch_fused.
+ * hf_plan_create + hf_launch_fused (hf_launch_fused_n for an entry of three kernels,
+ * whose lines carry three bounds and three block shapes).
  *
  * Plain C99 against include/hfuse_gfx950.h only (it doubles as the check that the
  * header is a C header).  Needs no GPU.
@@ -26,19 +27,22 @@ static const char *const kBarrier[] = {"none", "matched", "subset", "blockidx"};
 
 static int print_variant(const hf_config *cfg, int fusion, const char *file, const char *preset, int split_idx) {
   hf_plan *plan = NULL;
-  hf_partition p;
+  hf_partition_n p;
+  int k;
   int rc = hf_plan_create(cfg, fusion, preset, split_idx, 0, &plan);
   if (rc != HF_OK) {
     /* the reference prints the problem and goes on to the next variant (main.cpp:69-71) */
     printf("# %s\t%s\tidx %d\t%s\n", file, preset, split_idx, hf_last_error());
     return rc;
   }
-  rc = hf_plan_partition(plan, &p);
-  if (rc == HF_OK)
-    printf("%s\t%s\t%s\t%d\t[%u,%u)\t[%u,%u)\t%ux%ux%u\t%ux%ux%u\t%u\t%u\t%s\n", file, p.name, preset, split_idx,
-           p.lo[0], p.hi[0], p.lo[1], p.hi[1], p.block_dim[0].x, p.block_dim[0].y, p.block_dim[0].z,
-           p.block_dim[1].x, p.block_dim[1].y, p.block_dim[1].z, p.launch_threads, p.launch_blocks,
-           kBarrier[p.barrier_mode & 3]);
+  rc = hf_plan_partition_n(plan, &p);
+  if (rc == HF_OK) {
+    /* one bounds column and one block-shape column per kernel: two of each for a pair, three for a three-kernel entry */
+    printf("%s\t%s\t%s\t%d", file, p.name, preset, split_idx);
+    for (k = 0; k < p.n; k++) printf("\t[%u,%u)", p.lo[k], p.hi[k]);
+    for (k = 0; k < p.n; k++) printf("\t%ux%ux%u", p.block_dim[k].x, p.block_dim[k].y, p.block_dim[k].z);
+    printf("\t%u\t%u\t%s\n", p.launch_threads, p.launch_blocks, kBarrier[p.barrier_mode & 3]);
+  }
   hf_plan_free(plan);
   return rc;
 }
@@ -56,6 +60,7 @@ int main(int argc, char **argv) {
   }
   n = hf_config_num_fusions(cfg);
   printf("# file\tname\tpreset\tsplit_idx\tbounds1\tbounds2\tblockdim1\tblockdim2\tlaunch_threads\tlaunch_blocks\tbarrier\n");
+  printf("# (entries of three kernels: bounds1..3, blockdim1..3)\n");
   for (i = 0; i < n; i++) {
     const char *file = "", *k1 = "", *k2 = "";
     size_t pi;

@@ -43,6 +43,30 @@ def test_enumeration_matches_the_library(tool):
     assert all(r[1] == f"{r[1].split('_fused_kernel_')[0]}_fused_kernel_{r[2]}_idx_{r[3]}" for r in rows)
 
 
+def test_three_kernel_entries(tool):
+    """The shipped three-kernel list: every preset and split the driver's loop would print, three bounds a line."""
+    triples = os.path.join(PKG, "configs", "gfx950_triples.yaml")
+    out = subprocess.run([tool, triples, KERNELS], capture_output=True, text=True).stdout.splitlines()
+    rows = [ln.split("\t") for ln in out if not ln.startswith("#")]
+    cfg = H.Config.from_files(triples, KERNELS)
+    seen = 0
+    for i in range(cfg.num_fusions):
+        file = cfg.fusion(i)[0]
+        for preset in ("vfuse_lb", "vfuse", "hfuse", "hfuse_lb"):
+            idxs = range(cfg.num_splits(i)) if preset.startswith("hfuse") else [0]
+            for idx in idxs:
+                try:
+                    p = cfg.plan(i, preset, idx).partition_n
+                except hfuse_amd.HfuseError:
+                    continue      # printed as a comment line, as the reference prints the problem and goes on
+                want = [file, p.name.decode(), preset, str(idx)] + [f"[{p.lo[k]},{p.hi[k]})" for k in range(3)] + \
+                       ["x".join(str(v) for v in (p.block_dim[k].x, p.block_dim[k].y, p.block_dim[k].z)) for k in range(3)] + \
+                       [str(p.launch_threads), str(p.launch_blocks), BARRIER[p.barrier_mode]]
+                assert want in rows, want
+                seen += 1
+    assert seen >= 6 and len(rows) == seen
+
+
 def test_per_pair_table_and_errors(tool, tmp_path):
     table = tmp_path / "pair.yaml"
     table.write_text("- KernelName: im2col_kernel\n  HasBarriers: false\n  BlockDim:\n    X: 512\n    Y: 1\n    Z: 1\n"
