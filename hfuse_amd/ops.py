@@ -5,7 +5,7 @@ whose Python side calls each original kernel and each fused pair on torch tensor
 An `Op` is one original kernel bound to its inputs, with outputs allocated the way the PyTorch
 operator of the same name allocates them.  `run(op)` launches it natively; `run_fused(op1, op2)`
 launches both as one horizontally fused kernel (the pair must be in the fusion list, in either
-order).  Results are the op's outputs:
+order); `run_fused3(op0, op1, op2)` does the same for the reference's three-kernel lists.  Results are the op's outputs:
 
     from hfuse_amd import ops
     pooled, indices = ops.run(ops.max_pool2d(x, 3, 2, 1))
@@ -230,3 +230,31 @@ def run_fused(op1: Op, op2: Op, cfg: Optional[H.Config] = None, preset: str = "h
             grid = max(grid, (count + threads - 1) // threads)
     plan.launch(first.args, second.args, grid_blocks=grid, stream=stream)
     return op1.outputs, op2.outputs
+
+
+_default_triples: Optional[H.Config] = None
+
+
+def run_fused3(op0: Op, op1: Op, op2: Op, cfg: Optional[H.Config] = None, preset: str = "hfuse", stream=None):
+    """Launch three ops as one fused kernel; returns their outputs in the order given.
+
+    The three kernels must be an entry of `cfg` (default: the shipped three-kernel list, the reference's
+    configs/crypt_four.yaml, im2col_maxpool_norm.yaml and maxpool_summary_norm.yaml) in the entry's order."""
+    global _default_triples
+    if cfg is None:
+        if _default_triples is None:
+            from . import triples_config
+            _default_triples = triples_config()
+        cfg = _default_triples
+    trio = (op0, op1, op2)
+    index = cfg.find_fusion_n(*(op.kernel for op in trio))
+    plan = cfg.plan(index, preset)
+    part = plan.partition_n
+    grid = 0
+    for k, op in enumerate(trio):   # ethash: the grid times its share of the block covers the nonces
+        count = getattr(op, "count", 0)
+        if count:
+            threads = part.hi[k] - part.lo[k]
+            grid = max(grid, (count + threads - 1) // threads)
+    plan.launch_n([op.args for op in trio], grid_blocks=grid, stream=stream)
+    return tuple(op.outputs for op in trio)

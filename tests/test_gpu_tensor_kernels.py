@@ -777,6 +777,30 @@ def test_launches_can_be_captured_in_a_graph(cuda, cfg):
             t.check()                      # eager copies, comparisons and fills between the replays
 
 
+def test_three_kernel_launch_can_be_captured_in_a_graph(cuda):
+    """hf_launch_fused_n only enqueues one kernel as well: captured, then replayed three times with eager work between."""
+    import hfuse_amd
+    t = hfuse_amd.triples_config()
+    plan = t.plan(t.find_fusion_n("MaxPoolForward", "kernelHistogram1D", "batch_norm_collect_statistics_kernel"))
+    pool, hist, bn = MaxPool(cuda, 2, 4, 16, 16, (2, 2), (2, 2), (0, 0)), Histc(cuda, 50000), BnStats(cuda, 4, 9, 6, 6)
+    plan.launch_n([pool.args, hist.args, bn.args])   # warm-up outside the capture
+    sync()
+    side = torch.cuda.Stream()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.stream(side):
+        with torch.cuda.graph(graph, stream=side):
+            hist.out.zero_()                         # a fill kernel, not a memset node
+            plan.launch_n([pool.args, hist.args, bn.args])
+    for x in (pool, hist, bn):
+        x.check()
+    hist.out.fill_(3.0)
+    for replay in range(3):
+        graph.replay()
+        sync()
+        for x in (pool, hist, bn):
+            x.check()
+
+
 # ------------------------------------------------------------------ sizes at and beyond 2^31 elements
 # The general loops use 32-bit indices below 2^31 elements and 64-bit ones from there on.  These
 # cases sit above the limit; the expected values come from PyTorch's own GPU operators (at these

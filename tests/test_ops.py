@@ -105,3 +105,27 @@ def test_search_operators(cuda):
     ops.run_fused(e, b)
     assert ops.hits(e) == (want_n, [(h.nonce, h.digest_bytes(), h.mix_bytes()) for h in want_h])
     assert ops.hits(b)[0] == fb
+
+
+@pytest.mark.gpu
+def test_three_ops_in_one_launch(cuda):
+    """run_fused3 on the reference's im2col + max_pool2d + batch-norm list and on max_pool2d + histc + batch-norm."""
+    x, y, z = uniform((2, 8, 16, 16), 81), uniform((2, 8, 32, 32), 82), normal((4, 10, 7, 9), 83)
+    (col,), (val, idx), (mean, invstd) = ops.run_fused3(ops.im2col(x.to(cuda), 3, padding=1), ops.max_pool2d(y.to(cuda), 3, 2, 1),
+                                                        ops.batch_norm_collect_statistics(z.to(cuda), 1e-5))
+    torch.cuda.synchronize()
+    assert torch.equal(col.cpu(), F.unfold(x, 3, padding=1))
+    tv, ti = F.max_pool2d(y, 3, 2, 1, return_indices=True)
+    assert torch.equal(val.cpu(), tv) and torch.equal(idx.cpu(), ti)
+    wm, wi = torch_bn_stats(z, 1e-5)
+    assert rel_err(mean.cpu().numpy(), wm) < 1e-5 and rel_err(invstd.cpu().numpy(), wi) < 1e-5
+    h = uniform((50000,), 84, 0.0, 1.0)
+    (val, idx), (hist,), (mean, invstd) = ops.run_fused3(ops.max_pool2d(y.to(cuda), 2), ops.histc(h.to(cuda), 64, 0, 1),
+                                                         ops.batch_norm_collect_statistics(z.to(cuda), 1e-5), preset="vfuse")
+    torch.cuda.synchronize()
+    tv, ti = F.max_pool2d(y, 2, return_indices=True)
+    assert torch.equal(val.cpu(), tv) and torch.equal(idx.cpu(), ti)
+    assert torch.equal(hist.cpu(), torch.histc(h, 64, 0, 1))
+    assert rel_err(mean.cpu().numpy(), wm) < 1e-5
+    with pytest.raises(KeyError):
+        ops.run_fused3(ops.max_pool2d(y.to(cuda), 2), ops.im2col(x.to(cuda), 3), ops.histc(h.to(cuda), 64, 0, 1))
