@@ -7,6 +7,7 @@
 #include <cstring>
 #include <fstream>
 #include <initializer_list>
+#include <memory>
 #include <mutex>
 #include <new>
 #include <sstream>
@@ -719,31 +720,24 @@ HF_API int hf_plan_create(const hf_config *cfg, int fusion_index, const char *pr
     return fail(HF_EINVAL, "split_threads must be a multiple of the 64-lane wavefront");
   const FusionRow &f = cfg->cfg.fusions[fusion_index];
   if (f.kernels.size() != 2 && f.kernels.size() != 3) return unsupported_size(f);
-  auto plan = new hf_plan();
+  std::unique_ptr<hf_plan> plan(new hf_plan());  // freed on every early return and on an exception
   plan->preset = p;
   plan->n = (int)f.kernels.size();
   for (int i = 0; i < plan->n; i++) {
     plan->rows[i] = *cfg->cfg.find(f.kernels[i]);
-    if (!lookup_kernel(plan->rows[i].name, plan->ids[i])) {
-      int code = HF_ENOTFOUND;
-      std::string msg = "kernel '" + plan->rows[i].name + "' has no gfx950 implementation in this library";
-      delete plan;
-      return fail(code, msg);
-    }
+    if (!lookup_kernel(plan->rows[i].name, plan->ids[i]))
+      return fail(HF_ENOTFOUND, "kernel '" + plan->rows[i].name + "' has no gfx950 implementation in this library");
   }
   if (plan->n == 3) {
     // A three-kernel list: the Context's partition among three, no tuned keys, no lending, every
     // synchronising body on its own LDS arrival counter.
     if (is_crypto(plan->ids[0]) != is_crypto(plan->ids[1]) || is_crypto(plan->ids[0]) != is_crypto(plan->ids[2])) {
-      delete plan;
       return fail(HF_EUNSUPPORTED, "fusions mixing tensor kernels with search kernels are not built");
     }
     if (split_threads > 0) {
-      delete plan;
       return fail(HF_EINVAL, "split_threads shapes a pair; give a three-kernel plan its block with hf_plan_set_block_n");
     }
     if (f.split || f.threads || f.lending >= 0 || f.barrier >= 0 || f.launch_bound >= 0) {
-      delete plan;
       return fail(HF_EINVAL, "fusion '" + f.file + "': Split / Threads / Lending / Barrier / LaunchBound shape a pair; a three-kernel entry takes 'Blocks'");
     }
     // the entry's own block shape (`Blocks:`), applied like a pair's Split / Threads: to the table split of a horizontal preset
@@ -753,7 +747,6 @@ HF_API int hf_plan_create(const hf_config *cfg, int fusion_index, const char *pr
     for (int i = 0; own_shape && i < 3; i++) {
       if (shaped[i].block_dim.z != 1 || f.blocks[i] % shaped[i].block_dim.y) {
         std::string msg = "'Blocks' entry does not divide by BlockDim.Y of '" + shaped[i].name + "'";
-        delete plan;
         return fail(HF_EINVAL, msg);
       }
       shaped[i].block_dim.x = f.blocks[i] / shaped[i].block_dim.y;
@@ -770,17 +763,15 @@ HF_API int hf_plan_create(const hf_config *cfg, int fusion_index, const char *pr
       err3 = "search kernels are built for fused blocks of at most 512 threads";
     }
     if (rc3 != HF_OK) {
-      delete plan;
       return fail(rc3, err3);
     }
     plan->lending = false;
     plan->barrier_mode = (body_has_barriers(plan->ids[0]) || body_has_barriers(plan->ids[1]) || body_has_barriers(plan->ids[2]))
                              ? HF_BARRIER_SUBSET : HF_BARRIER_NONE;
-    *out = plan;
+    *out = plan.release();
     return HF_OK;
   }
   if (is_crypto(plan->ids[0]) != is_crypto(plan->ids[1])) {
-    delete plan;
     return fail(HF_EUNSUPPORTED, "pairs mixing a tensor kernel with a search kernel are not built");
   }
   std::string err;
@@ -790,19 +781,16 @@ HF_API int hf_plan_create(const hf_config *cfg, int fusion_index, const char *pr
   if (tuned && f.threads == 0) split_threads = (int)f.split;
   int rc = make_partition(plan->rows[0], plan->rows[1], *p, split_idx, split_threads, plan->part, err);
   if (rc != HF_OK) {
-    delete plan;
     return fail(rc, err);
   }
   if (tuned && f.threads > 0) {
     // the pair's tuned block shape from the fusion list: Split threads of kernel 1 in a block of Threads
-    rc = hf_plan_set_block(plan, (int)f.split, (int)(f.threads - f.split));
+    rc = hf_plan_set_block(plan.get(), (int)f.split, (int)(f.threads - f.split));
     if (rc != HF_OK) {
-      delete plan;
       return rc;
     }
   }
   if (is_crypto(plan->ids[0]) && !p->base_line && plan->part.launch_threads > 512) {
-    delete plan;
     return fail(HF_EINVAL, "search kernels are built for fused blocks of at most 512 threads");
   }
   if (f.lending >= 0) plan->lending = f.lending != 0;
@@ -814,13 +802,12 @@ HF_API int hf_plan_create(const hf_config *cfg, int fusion_index, const char *pr
   // also share the hardware barrier: HF_BARRIER_MATCHED via hf_plan_set_barrier_mode.)
   plan->barrier_mode = (b1 || b2) ? HF_BARRIER_SUBSET : HF_BARRIER_NONE;
   if (f.barrier >= 0 && !p->base_line) {
-    rc = hf_plan_set_barrier_mode(plan, f.barrier);
+    rc = hf_plan_set_barrier_mode(plan.get(), f.barrier);
     if (rc != HF_OK) {
-      delete plan;
       return rc;
     }
   }
-  *out = plan;
+  *out = plan.release();
   return HF_OK;
 } catch (...) {
   return trap_exception();
@@ -1280,6 +1267,35 @@ HF_API int hf_launch_fused(const hf_plan *plan, const void *args1, const void *a
   return trap_exception();
 }
 
+extern "C++" {
+namespace {
+// `warmup` untimed repetitions of once(r), then `iters` timed ones between two HIP events recorded on `stream`.
+template <class Once>
+int time_repetitions(hipStream_t stream, int warmup, int iters, Once once, float *elapsed_ms) {
+  for (int r = 0; r < warmup; r++) {
+    int rc = once(r);
+    if (rc != HF_OK) return rc;
+  }
+  hipEvent_t t0, t1;
+  hipError_t e = hipEventCreate(&t0);
+  if (e != hipSuccess) return hip_fail(e, "hipEventCreate");
+  e = hipEventCreate(&t1);
+  if (e != hipSuccess) { (void)hipEventDestroy(t0); return hip_fail(e, "hipEventCreate"); }
+  int rc = HF_OK;
+  e = hipEventRecord(t0, stream);
+  for (int r = 0; r < iters && rc == HF_OK && e == hipSuccess; r++) rc = once(warmup + r);
+  if (e == hipSuccess) e = hipEventRecord(t1, stream);
+  if (e == hipSuccess) e = hipEventSynchronize(t1);
+  if (e == hipSuccess) e = hipEventElapsedTime(elapsed_ms, t0, t1);
+  (void)hipEventDestroy(t0);
+  (void)hipEventDestroy(t1);
+  if (rc != HF_OK) return rc;
+  if (e != hipSuccess) return hip_fail(e, "timing");
+  return HF_OK;
+}
+}  // namespace
+}  // extern "C++"
+
 HF_API int hf_time_pair(const hf_plan *plan, int mode, const void *const *args1, const void *const *args2, int nsets,
                         int first_set, int warmup, int iters, int grid_blocks, void *stream_, float *elapsed_ms) try {
   if (!plan || !args1 || !args2 || !elapsed_ms) return fail(HF_EINVAL, "null argument");
@@ -1340,26 +1356,7 @@ HF_API int hf_time_pair(const hf_plan *plan, int mode, const void *const *args1,
     }
     return rc;
   };
-  for (int i = 0; i < warmup; i++) {
-    int rc = once(i);
-    if (rc != HF_OK) return rc;
-  }
-  hipEvent_t t0, t1;
-  hipError_t e = hipEventCreate(&t0);
-  if (e != hipSuccess) return hip_fail(e, "hipEventCreate");
-  e = hipEventCreate(&t1);
-  if (e != hipSuccess) { (void)hipEventDestroy(t0); return hip_fail(e, "hipEventCreate"); }
-  int rc = HF_OK;
-  e = hipEventRecord(t0, stream);
-  for (int i = 0; i < iters && rc == HF_OK && e == hipSuccess; i++) rc = once(warmup + i);
-  if (e == hipSuccess) e = hipEventRecord(t1, stream);
-  if (e == hipSuccess) e = hipEventSynchronize(t1);
-  if (e == hipSuccess) e = hipEventElapsedTime(elapsed_ms, t0, t1);
-  (void)hipEventDestroy(t0);
-  (void)hipEventDestroy(t1);
-  if (rc != HF_OK) return rc;
-  if (e != hipSuccess) return hip_fail(e, "timing");
-  return HF_OK;
+  return time_repetitions(stream, warmup, iters, once, elapsed_ms);
 } catch (...) {
   return trap_exception();
 }
@@ -1435,26 +1432,7 @@ HF_API int hf_time_fused_n(const hf_plan *plan, int mode, const void *const *arg
     }
     return HF_OK;
   };
-  for (int r = 0; r < warmup; r++) {
-    int rc = once(r);
-    if (rc != HF_OK) return rc;
-  }
-  hipEvent_t t0, t1;
-  hipError_t e = hipEventCreate(&t0);
-  if (e != hipSuccess) return hip_fail(e, "hipEventCreate");
-  e = hipEventCreate(&t1);
-  if (e != hipSuccess) { (void)hipEventDestroy(t0); return hip_fail(e, "hipEventCreate"); }
-  int rc = HF_OK;
-  e = hipEventRecord(t0, stream);
-  for (int r = 0; r < iters && rc == HF_OK && e == hipSuccess; r++) rc = once(warmup + r);
-  if (e == hipSuccess) e = hipEventRecord(t1, stream);
-  if (e == hipSuccess) e = hipEventSynchronize(t1);
-  if (e == hipSuccess) e = hipEventElapsedTime(elapsed_ms, t0, t1);
-  (void)hipEventDestroy(t0);
-  (void)hipEventDestroy(t1);
-  if (rc != HF_OK) return rc;
-  if (e != hipSuccess) return hip_fail(e, "timing");
-  return HF_OK;
+  return time_repetitions(stream, warmup, iters, once, elapsed_ms);
 } catch (...) {
   return trap_exception();
 }
