@@ -38,6 +38,18 @@ int main(int argc, char **argv) {
     if (!parse_config((rng() % 16 == 0) ? nullptr : f.c_str(), k.c_str(), cfg, err)) { bad++; continue; }
     ok++;
     for (auto &fr : cfg.fusions) {
+      if (fr.kernels.size() == 3) {   // the Context's partition among three, every preset and split
+        const KernelRow *r3[3] = {cfg.find(fr.kernels[0]), cfg.find(fr.kernels[1]), cfg.find(fr.kernels[2])};
+        if (!r3[0] || !r3[1] || !r3[2]) continue;
+        for (const char *pn : {"hfuse", "hfuse_lb", "vfuse", "vfuse_lb"}) {
+          for (int idx = -2; idx < 12; idx++) {
+            Partition part; std::string e3;
+            if (make_partition_n(r3, 3, *find_preset(pn), idx, part, e3) == 0)
+              for (int h = 0; h < 3; h++) if (part.hi[h] > part.lo[h]) { (void)local_index(part.lo[h], part.lo[h], part.block_dim[h]); (void)local_index(part.hi[h] - 1, part.lo[h], part.block_dim[h]); }
+          }
+        }
+        continue;
+      }
       if (fr.kernels.size() != 2) continue;
       const KernelRow *a = cfg.find(fr.kernels[0]), *b = cfg.find(fr.kernels[1]);
       if (!a || !b) continue;

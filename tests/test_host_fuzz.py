@@ -23,10 +23,11 @@ def fuzzer(tmp_path_factory):
     return exe
 
 
+@pytest.mark.parametrize("fusion", ["gfx950_fusion.yaml", "gfx950_triples.yaml"])
 @pytest.mark.parametrize("maxmut", [1, 6])
-def test_mutated_configs_never_crash_the_host_model(fuzzer, maxmut):
+def test_mutated_configs_never_crash_the_host_model(fuzzer, maxmut, fusion):
     env = dict(os.environ, MAXMUT=str(maxmut))
-    r = subprocess.run([fuzzer, os.path.join(PKG, "configs", "gfx950_fusion.yaml"),
+    r = subprocess.run([fuzzer, os.path.join(PKG, "configs", fusion),
                         os.path.join(PKG, "configs", "gfx950_kernels.yaml"), "12000"],
                        capture_output=True, text=True, env=env, timeout=300)
     assert r.returncode == 0, r.stderr[-2000:]
