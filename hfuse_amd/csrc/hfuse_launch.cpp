@@ -1,7 +1,7 @@
 // hfuse-launch: a C++ host program over the C-ABI, the shape of the callers the reference's
 // kernels were generated for (its README's TorchKernel extension and ethminer's fuse/fuser):
-// for one pair of the fusion list it launches native kernel 1, native kernel 2, both back to
-// back and the fused kernel on identical synthetic inputs, several times in one process,
+// for one pair (or three-kernel entry) of the fusion list it launches native kernel 1, native kernel 2,
+// both back to back and the fused kernel on identical synthetic inputs, several times in one process,
 // prints the per-launch durations, and checks that the fused launch produced the same bytes
 // as the two native launches (batch-norm statistics: the same values to 1e-5 relative).
 //
@@ -205,7 +205,7 @@ std::unique_ptr<Workload> make_workload(const std::string &k, bool second_of_his
       Buffer *dag = add(w->inputs, (size_t)items * 128);
       hf_check(hf_fill_splitmix64(static_cast<uint64_t *>(dag->dev), (uint64_t)items * 16, seed, nullptr));
       hip_check(hipDeviceSynchronize(), "dag fill");
-      hf_check(hf_ethash_set_constants(dag->dev, items, header, small ? (1ull << 56) - 1 : (1ull << 44) - 1, nullptr));
+      hf_check(hf_ethash_set_constants(dag->dev, items, header, small ? (1ull << 54) - 1 : (1ull << 44) - 1, nullptr));   // about 16 hits either way: well under the record's 64 slots
       hf_ethash_args a[2] = {{static_cast<hf_search_results *>(res[0]->dev), 0}, {static_cast<hf_search_results *>(res[1]->dev), 0}};
       w->set_args(a[0], a[1]);
       w->grid = (int)(threads / 128);
@@ -300,6 +300,55 @@ double run_pair(hf_config *cfg, int index, const std::string &preset, int split,
   return speedup;
 }
 
+// A three-kernel entry (the reference's configs/crypt_four.yaml, im2col_maxpool_norm.yaml, maxpool_summary_norm.yaml):
+// the three native kernels, then the one fused kernel, on identical inputs; outputs compared; both forms timed.
+double run_triple(hf_config *cfg, int index, const std::string &preset, int split, int iters, bool small, bool &ok) {
+  const char *names[3] = {"", "", ""};
+  for (int k = 0; k < 3; k++) hf_check(hf_config_fusion_kernel(cfg, index, k, &names[k]));
+  hf_plan *plan = nullptr;
+  hf_check(hf_plan_create(cfg, index, preset.c_str(), split, 0, &plan));
+  hf_partition_n part;
+  hf_check(hf_plan_partition_n(plan, &part));
+  std::printf("%s + %s + %s as %s (%u threads: [%u,%u) + [%u,%u) + [%u,%u))\n", names[0], names[1], names[2], part.name,
+              part.launch_threads, part.lo[0], part.hi[0], part.lo[1], part.hi[1], part.lo[2], part.hi[2]);
+  bool with_hist = false;
+  for (int k = 0; k < 3; k++) with_hist = with_hist || std::string(names[k]) == "kernelHistogram1D";
+  std::unique_ptr<Workload> w[3];
+  int native_grid = 0, fused_grid = 0;
+  for (int k = 0; k < 3; k++) {
+    w[k] = make_workload(names[k], with_hist && std::string(names[k]) == "MaxPoolForward", small, 0x48467573ull + k);
+    if (w[k]->grid) {   // ethash scans grid * (its block) nonces: natively 128-thread blocks, fused its share of the block
+      native_grid = w[k]->grid;
+      fused_grid = (int)(w[k]->hashes / (part.hi[k] - part.lo[k]));
+    }
+    w[k]->reset();
+  }
+  hip_check(hipDeviceSynchronize(), "reset");
+  const void *fused_args[3], *native_args[3];
+  for (int k = 0; k < 3; k++) {
+    hf_check(hf_launch_native(names[k], w[k]->args_native.data(), w[k]->grid, 0, nullptr));
+    fused_args[k] = w[k]->args_fused.data();
+    native_args[k] = w[k]->args_native.data();
+  }
+  hf_check(hf_launch_fused_n(plan, fused_args, 3, fused_grid, nullptr));
+  hip_check(hipDeviceSynchronize(), "compared launches");
+  ok = true;
+  for (int k = 0; k < 3; k++) {
+    const bool same = same_outputs(*w[k]);
+    std::printf("fused == native: %s %s\n", names[k], same ? "yes" : "NO");
+    ok = ok && same;
+  }
+  float ms[2];
+  hf_check(hf_time_fused_n(plan, 2, native_args, 3, 1, 0, 2, iters, native_grid, nullptr, &ms[0]));
+  hf_check(hf_time_fused_n(plan, 3, native_args, 3, 1, 0, 2, iters, fused_grid, nullptr, &ms[1]));
+  std::printf("%-60s %10.3f us per launch\n", "three native launches back to back", 1e3 * ms[0] / iters);
+  std::printf("%-60s %10.3f us per launch\n", part.name, 1e3 * ms[1] / iters);
+  const double speedup = (ms[0] / ms[1] - 1.0) * 100.0;
+  std::printf("speedup of the fused kernel over back to back: %+.1f %%\n", speedup);
+  hf_plan_free(plan);
+  return speedup;
+}
+
 }  // namespace
 
 int main(int argc, char **argv) {
@@ -327,7 +376,8 @@ int main(int argc, char **argv) {
     for (int i = 0; i < n; i++) {
       const char *file = "", *k1 = "", *k2 = "";
       hf_check(hf_config_fusion(cfg, i, &file, &k1, &k2));
-      if (which == "all" ? hf_config_fusion_size(cfg, i) == 2 : (which == file || std::to_string(i) == which)) {
+      const int size = hf_config_fusion_size(cfg, i);
+      if (which == "all" ? (size == 2 || size == 3) : (which == file || std::to_string(i) == which)) {
         todo.push_back(i);
         if (which != "all") break;
       }
@@ -337,7 +387,8 @@ int main(int argc, char **argv) {
     std::vector<std::pair<std::string, double>> summary;
     for (int index : todo) {
       bool ok = false;
-      const double speedup = run_pair(cfg, index, preset, split, iters, small, ok);
+      const double speedup = hf_config_fusion_size(cfg, index) == 3 ? run_triple(cfg, index, preset, split, iters, small, ok)
+                                                                   : run_pair(cfg, index, preset, split, iters, small, ok);
       all_ok = all_ok && ok;
       const char *file = "", *k1 = "", *k2 = "";
       hf_check(hf_config_fusion(cfg, index, &file, &k1, &k2));

@@ -45,6 +45,16 @@ def test_all_pairs_in_one_run(cuda):
     assert " NO" not in r.stdout and "fused over back to back" in r.stdout
 
 
+def test_three_kernel_list_small(cuda):
+    cfg = hfuse_amd.triples_config()
+    triples = os.path.join(PKG, "configs", "gfx950_triples.yaml")
+    assert os.path.exists(TOOL), "build the library first (make -C hfuse_amd/csrc)"
+    r = subprocess.run([TOOL, triples, KERNELS, "all", "--small", "--iters", "2"], capture_output=True, text=True, timeout=300)
+    assert r.returncode == 0, (r.stdout[-2000:], r.stderr)
+    assert r.stdout.count("fused == native:") == 3 * cfg.num_fusions
+    assert " NO" not in r.stdout and "three native launches back to back" in r.stdout
+
+
 def test_errors(cuda):
     assert run("NoSuchPair").returncode == 1
     assert run("0", "--preset", "hfuse_bar_sync").returncode == 1
