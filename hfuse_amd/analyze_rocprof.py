@@ -9,7 +9,8 @@ without launch bounds; scripts/analyze_nvprof.py:650-690) and two tables of metr
 rocprofv3 names a launch by its HIP symbol, so the tag comes from the kernel template and the
 block shape instead:
 
-    native_kernel<XBody, ...>            ST   one original kernel
+    native_kernel<XBody, ...>            ST   one original kernel (native_kernel_capped: the same with its
+                                              residency capped, as im2col is launched)
     vertical_kernel<XBody, YBody, ...>   VF   the same threads run both bodies
     fused_kernel<XBody, YBody, .., 0>    HF   horizontally fused, tagged with the workgroup size
     fused_kernel<XBody, YBody, .., 1>    HF+M the same with the shared hardware barrier
@@ -58,7 +59,7 @@ SHORT = {
 }
 TAG_ORDER = ("ST", "VF", "VF-LB", "HF", "HF-LB", "HF+M", "HF+M-LB", "BI")
 
-_TEMPLATE = re.compile(r"hfuse::(native_kernel|fused_kernel_lb|fused_kernel|vertical_kernel_lb|vertical_kernel|blockidx_kernel)<(.*)>\(")
+_TEMPLATE = re.compile(r"hfuse::(native_kernel_capped|native_kernel|fused_kernel_lb|fused_kernel|vertical_kernel_lb|vertical_kernel|blockidx_kernel)<(.*)>\(")
 _BODY = re.compile(r"hfuse::(\w+Body(?:<[^<>]*>)?)")
 
 
@@ -81,7 +82,7 @@ def parse_kernel_name(name: str) -> Optional[Tuple[str, Tuple[str, ...]]]:
     bodies = [BODY_TO_KERNEL.get(b) for b in _BODY.findall(params)]
     if not bodies or any(b is None for b in bodies):
         return None
-    if kind == "native_kernel":
+    if kind in ("native_kernel", "native_kernel_capped"):
         return "ST", (bodies[0],)
     if len(bodies) != 2:
         return None

@@ -19,6 +19,8 @@
 #pragma once
 #include <hip/hip_runtime.h>
 
+#include <type_traits>
+
 namespace hfuse {
 
 typedef float f32x4 __attribute__((ext_vector_type(4)));
@@ -120,6 +122,28 @@ __global__ __launch_bounds__(T) void native_kernel(typename K::Args a, unsigned 
                              bid * blockDim.x, gridDim.x * blockDim.x};
   K::run(a, sb, smem, hint);
 }
+
+// The same with residency capped at W waves per SIMD (the register allocation is padded so that no
+// more fit).  A body asks for it with `kNativeWaves`: a kernel that writes many separate streams per
+// work item runs faster when fewer of its waves write at once.
+template <class K, int T, int W>
+__global__ __launch_bounds__(T) __attribute__((amdgpu_waves_per_eu(W, W))) void native_kernel_capped(typename K::Args a,
+                                                                                                   unsigned hint) {
+  extern __shared__ __align__(16) unsigned char smem[];
+  const unsigned bid = blockIdx.x;
+  SubBlock<BAR_WORKGROUP> sb{threadIdx.x, blockDim.x, bid, gridDim.x, nullptr, 0,
+                             bid * blockDim.x, gridDim.x * blockDim.x};
+  K::run(a, sb, smem, hint);
+}
+
+template <class K, class = void>
+struct NativeWaves {
+  static constexpr int value = 0;  // no cap
+};
+template <class K>
+struct NativeWaves<K, std::void_t<decltype(K::kNativeWaves)>> {
+  static constexpr int value = K::kNativeWaves;
+};
 
 // Horizontal fusion: waves [0, d1/64) run kernel 1, the rest run kernel 2.  The
 // selector is a scalar (readfirstlane) so each wave takes one side without

@@ -12,8 +12,13 @@ constexpr int kDlBlock = 1024;  // launch bound: any split with d1 + d2 <= 1024
 
 template <class K>
 hipError_t dl_native(const void *args, unsigned hint, unsigned grid, unsigned block, size_t lds, hipStream_t s) {
-  hipLaunchKernelGGL((native_kernel<K, kDlBlock>), dim3(grid), dim3(block), lds, s,
-                     *static_cast<const typename K::Args *>(args), hint);
+  constexpr int kWaves = NativeWaves<K>::value;
+  if constexpr (kWaves != 0)
+    hipLaunchKernelGGL((native_kernel_capped<K, kDlBlock, kWaves>), dim3(grid), dim3(block), lds, s,
+                       *static_cast<const typename K::Args *>(args), hint);
+  else
+    hipLaunchKernelGGL((native_kernel<K, kDlBlock>), dim3(grid), dim3(block), lds, s,
+                       *static_cast<const typename K::Args *>(args), hint);
   return hipGetLastError();
 }
 

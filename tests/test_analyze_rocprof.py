@@ -15,6 +15,8 @@ TRACE_COLS = ["Kind", "Kernel_Name", "Start_Timestamp", "End_Timestamp", "VGPR_C
 
 def test_parse_kernel_name():
     assert A.parse_kernel_name(N.format(b="Im2colBody")) == ("ST", ("im2col_kernel",))
+    capped = "void hfuse::native_kernel_capped<hfuse::Im2colBody, 1024, 4>(hfuse::Im2colBody::Args, unsigned int)"
+    assert A.parse_kernel_name(capped) == ("ST", ("im2col_kernel",))
     assert A.parse_kernel_name(F.format(a="HistcBody", b="MaxPoolBody", m="false")) == ("HF", ("kernelHistogram1D", "MaxPoolForward"))
     assert A.parse_kernel_name(F.format(a="BnStatsBody", b="HistcBody", m="true"))[0] == "HF+M"
     assert A.parse_kernel_name(V.format(a="EthashBody", b="Blake2bBody<4, false>")) == ("VF", ("ethash_search", "sia_blake2b_gpu_hash"))

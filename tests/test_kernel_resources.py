@@ -37,7 +37,8 @@ def test_library_holds_gfx950_code_objects():
 def test_every_kernel_family_is_present(rows):
     names = [short_name(r.name) for r in rows]
     for body in TENSOR + SEARCH:
-        assert any(n.startswith("native_kernel<" + body) for n in names), body
+        # (im2col's native kernel is the build with its residency capped)
+        assert any(n.startswith(("native_kernel<" + body, "native_kernel_capped<" + body)) for n in names), body
     for kind in ("fused_kernel<", "vertical_kernel<", "blockidx_kernel<", "fused_kernel_lb<", "vertical_kernel_lb<"):
         assert sum(n.startswith(kind) for n in names) >= 20, kind
 
@@ -65,7 +66,7 @@ def test_fusing_never_halves_occupancy(rows):
     """A fused kernel needs about the registers of its hungrier half, not more than 1.25x."""
     native = {}
     for r in rows:
-        m = re.match(r"native_kernel<(.+), \d+>$", short_name(r.name))
+        m = re.match(r"native_kernel(?:_capped)?<(.+?), \d+(?:, \d+)?>$", short_name(r.name))
         if m:
             native[m.group(1)] = r
     checked = 0
