@@ -45,16 +45,21 @@ enum KernelId {
   K_COUNT
 };
 
-// Register-bounded builds.  Every pair has one for kBoundedWaves waves per SIMD; the benchmarked
-// pairs whose occupancy formula (min over the kernels of regfile / Reg / threads, capped by the
+// Register-bounded builds.  Every pair has one for kBoundedWaves waves per SIMD; the pairs of the
+// shipped list whose occupancy formula (min over the kernels of regfile / Reg / threads, capped by the
 // resident threads: lib/KernelFuser/KernelPrinter.cpp:44-66, with this part's 128 K registers and
-// 2048 threads per CU) asks for fewer waves have a second build at exactly that bound.
+// 2048 threads per CU) asks for fewer waves at their shipped block shape have a second build at exactly
+// that bound.
 constexpr int kBoundedWaves = 8;
 constexpr int pair_extra_waves(KernelId k1, KernelId k2) {
-  return (k1 == K_IM2COL && k2 == K_MAXPOOL) ? 5      // 2 blocks of 256 + 448 threads
-         : (k1 == K_HISTC && k2 == K_MAXPOOL) ? 7     // 2 blocks of 768 + 128
-         : (k1 == K_ETHASH && k2 == K_SIA_BLAKE2B) ? 6  // 8 blocks of 128 + 64
-                                                   : 0;
+  return (k1 == K_IM2COL && k2 == K_MAXPOOL) ? 5                // 2 blocks of 256 + 448 threads
+         : (k1 == K_HISTC && k2 == K_MAXPOOL) ? 7               // 2 blocks of 768 + 128
+         : (k1 == K_ETHASH && k2 == K_SIA_BLAKE2B) ? 6          // 8 blocks of 128 + 64
+         : (k1 == K_IM2COL && k2 == K_HISTC) ? 7                // 2 blocks of 640 + 256
+         : (k1 == K_IM2COL && k2 == K_UPSAMPLE_NEAREST) ? 6     // 2 blocks of 256 + 512
+         : (k1 == K_MAXPOOL && k2 == K_BNSTATS) ? 7             // 9 blocks of 64 + 128
+         : (k1 == K_IM2COL && k2 == K_UPSAMPLE_BILINEAR) ? 6    // 2 blocks of 256 + 512
+                                                         : 0;
 }
 // The bound of the build that runs when `waves` waves per SIMD are asked for (0: the plain build).
 constexpr int built_bound_waves(KernelId k1, KernelId k2, int waves) {

@@ -456,14 +456,22 @@ def test_fused_histc_maxpool_full_benchmark_size(cuda, cfg):
 
 
 def test_bounded_builds_at_every_wave_count(cuda, cfg):
-    """The register-bounded builds of the benchmarked tensor pairs -- at the occupancy formula's own value
-    (5 and 7 waves per SIMD) and at 8 -- give the same bits as the plain build."""
+    """The register-bounded builds of the shipped thread partitions -- at the occupancy formula's own value
+    (5, 6 and 7 waves per SIMD) and at 8 -- give the same bits as the plain build."""
     cases = [("im2col_kernel", "MaxPoolForward", lambda: Im2col(cuda, 4, 16, 56, 56),
               lambda: MaxPool(cuda, 4, 16, 112, 112, (3, 3), (2, 2), (1, 1)), 5),
              ("kernelHistogram1D", "MaxPoolForward", lambda: Histc(cuda, 1 << 20),
               lambda: MaxPool(cuda, 4, 32, 64, 64, (2, 2), (2, 2), (0, 0)), 7),
              ("batch_norm_collect_statistics_kernel", "upsample_nearest2d_out_frame", lambda: BnStats(cuda, 8, 32, 28, 28),
-              lambda: Upsample(cuda, 8, 16, 56, 56, (112, 112)), 8)]
+              lambda: Upsample(cuda, 8, 16, 56, 56, (112, 112)), 8),
+             # the other shipped thread partitions whose formula gives fewer than 8
+             ("im2col_kernel", "upsample_nearest2d_out_frame", lambda: Im2col(cuda, 4, 16, 56, 56),
+              lambda: Upsample(cuda, 8, 16, 56, 56, (112, 112)), 6),
+             ("im2col_kernel", "kernelHistogram1D", lambda: Im2col(cuda, 4, 16, 56, 56), lambda: Histc(cuda, 1 << 20), 7),
+             ("MaxPoolForward", "batch_norm_collect_statistics_kernel",
+              lambda: MaxPool(cuda, 4, 16, 112, 112, (3, 3), (2, 2), (1, 1)), lambda: BnStats(cuda, 8, 32, 28, 28), 7),
+             ("im2col_kernel", "upsample_bilinear2d_out_frame", lambda: Im2col(cuda, 4, 16, 56, 56),
+              lambda: Bilinear(cuda, 4, 16, 56, 56, (112, 112)), 6)]
     for k1, k2, m1, m2, formula in cases:
         plan = cfg.plan(cfg.find_fusion(k1, k2), "hfuse_lb")
         assert plan.launch_waves == (formula, formula)

@@ -550,10 +550,18 @@ def test_launch_bound_formula_and_built_variants(cfg):
         plain.set_barrier_mode(L.HF_BARRIER_BLOCKIDX)
         plain.set_launch_bound(True)
         assert plain.launch_waves[1] == 0                                 # the block-index partition has no bounded build
-    # pairs beyond the benchmarked five have the 8-wave build only
-    i = cfg.find_fusion("im2col_kernel", "upsample_nearest2d_out_frame")
-    p = cfg.plan(i, "hfuse_lb")
-    p.set_launch_bound(True)
+    # beyond the benchmarked five: the shipped thread partitions whose formula gives fewer than 8 waves have a build at
+    # that value too -- im2col(42, 256) + upsample(22, 512): min(12, 11, 2) = 2 blocks of 768 threads = 6 waves per SIMD
+    for k1, k2, w in (("im2col_kernel", "upsample_nearest2d_out_frame", 6), ("im2col_kernel", "kernelHistogram1D", 7),
+                      ("MaxPoolForward", "batch_norm_collect_statistics_kernel", 7),
+                      ("im2col_kernel", "upsample_bilinear2d_out_frame", 6)):
+        p = cfg.plan(cfg.find_fusion(k1, k2), "hfuse_lb")
+        assert p.launch_waves == (w, w), (k1, k2, p.launch_waves)
+        p.set_launch_waves(8)
+        assert p.launch_waves == (w, 8)
+    # every other pair has the 8-wave build only
+    p = cfg.plan(cfg.find_fusion("upsample_nearest2d_out_frame", "batch_norm_collect_statistics_kernel"), "hfuse_lb")
+    p.set_launch_waves(3)
     assert p.launch_waves[1] == 8
 
 
