@@ -51,6 +51,16 @@ OPS_SHA256D = 4336
 OPS_BLAKE2B = 2528
 ETHASH_BYTES = 8192               # 64 accesses x 128 bytes of DAG per hash
 
+# What a fused tensor pair could reach at best: its bytes at the rates bare loops reach on this part (16-byte
+# non-temporal accesses over 512 MiB: reads 7.1 TB/s, writes 6.5 TB/s), reads and writes after each other with no
+# turnaround cost, plus the 1.7 us an empty kernel takes.  (read bytes, written bytes) of both kernels of a pair:
+READ_GBPS_MEASURED, WRITE_GBPS_MEASURED, EMPTY_LAUNCH_US = 7100.0, 6500.0, 1.7
+PAIR_READ_WRITE_BYTES = {
+    "im2col_maxpool": (4 * 32 * 64 * (56 * 56 + 112 * 112), 4 * 32 * 576 * 3136 + 12 * 32 * 64 * 56 * 56),
+    "bn_upsample": (4 * 32 * 256 * 28 * 28 + 4 * 32 * 64 * 56 * 56, 2 * 4 * 256 + 4 * 32 * 64 * 112 * 112),
+    "histc_maxpool": (4 * (1 << 26) + 4 * 16 * 128 * 64 * 64, 4 * 1024 + 12 * 16 * 128 * 32 * 32),
+}
+
 TENSOR_NAMES = ("im2col_maxpool", "bn_upsample", "histc_maxpool")
 SEARCH_NAMES = ("sha256d_blake2b", "ethash_blake2b")
 MODE_KEYS = {0: "t_a_ms", 1: "t_b_ms", 2: "t_b2b_ms", 3: "t_fused_ms", 4: "t_two_streams_ms"}
@@ -523,6 +533,11 @@ def main():
             r["a_gbps"] = pair.bytes1 / (r["t_a_ms"] * 1e-3) / 1e9
             r["b_gbps"] = pair.bytes2 / (r["t_b_ms"] * 1e-3) / 1e9
             judge(r)
+            rd, wr = PAIR_READ_WRITE_BYTES[name]
+            floor_ms = (rd / READ_GBPS_MEASURED + wr / WRITE_GBPS_MEASURED) * 1e-6 + EMPTY_LAUNCH_US * 1e-3
+            r["streaming_bound"] = {"fused_floor_ms": floor_ms, "max_speedup_pct": (r["t_b2b_ms"] / floor_ms - 1.0) * 100.0,
+                                    "fused_over_floor": r["t_fused_ms"] / floor_ms,
+                                    "basis": "read bytes at 7.1 TB/s + written bytes at 6.5 TB/s (bare loops on this part) + 1.7 us launch"}
         if name == args.headline:
             r["wall_ms_per_step"], r["event_ms_per_step"] = timed_region(plan, pair)
         r["check"] = check_tensor_pair(name, pair, plan)

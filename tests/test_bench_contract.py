@@ -58,3 +58,6 @@ def test_roofline_constants(bench):
                    "histc_maxpool": 268_439_552 + 58_720_256, "ethash_blake2b": (1 << 28) * 8192}
     for name, measured in bench.TRAFFIC_BYTES.items():
         assert 0.98 < measured / algorithmic[name] < 1.02, name
+    # read + written bytes of a tensor pair are its algorithmic bytes
+    for name, (rd, wr) in bench.PAIR_READ_WRITE_BYTES.items():
+        assert rd + wr == algorithmic[name], name
