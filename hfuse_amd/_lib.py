@@ -14,6 +14,7 @@ LIB_PATH = os.path.join(_HERE, "libhfuse_gfx950.so")
 HF_OK, HF_EINVAL, HF_EPARSE, HF_ENOTFOUND, HF_EUNSUPPORTED, HF_EHIP, HF_EIO, HF_ENOMEM = 0, -1, -2, -3, -4, -5, -6, -7
 HF_BARRIER_NONE, HF_BARRIER_MATCHED, HF_BARRIER_SUBSET, HF_BARRIER_BLOCKIDX = 0, 1, 2, 3
 HF_SPLIT_TABLE, HF_SPLIT_EXECTIME = -1, -2
+ABI_VERSION = 300          # what hf_version() of a matching library answers
 HF_MAX_SEARCH_RESULTS = 64
 HF_MAX_TENSORINFO_DIMS = 8
 
@@ -196,6 +197,10 @@ def lib() -> C.CDLL:
             fn = getattr(handle, name)
             fn.restype = restype
             fn.argtypes = argtypes
+        # signatures changed between versions (hf_time_pair gained an argument): a stale build would take shifted arguments
+        if handle.hf_version() != ABI_VERSION:
+            raise ImportError(f"{LIB_PATH} answers hf_version() = {handle.hf_version()}, this package binds version "
+                              f"{ABI_VERSION}: rebuild it (`make -C hfuse_amd/csrc`)")
         _lib = handle
     return _lib
 

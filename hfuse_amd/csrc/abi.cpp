@@ -410,7 +410,9 @@ int prepare_histc(const hf_histc_args &a, Prepared &p) {
   std::memcpy(p.blob, &a, sizeof a);
   // contiguous input: 16-byte loads from the first aligned element on; the up to three elements
   // before it (HINT_HIST_HEAD bits) and the tail go through scalar loads
-  const bool fast = a.b.strides[0] == 1 && (reinterpret_cast<uintptr_t>(a.b.data) & 3u) == 0;
+  // (the vector path numbers its 1-2 KiB chunks in 32 bits: inputs below 2^40 elements, far more than HBM holds)
+  const bool fast = a.b.strides[0] == 1 && (reinterpret_cast<uintptr_t>(a.b.data) & 3u) == 0 &&
+                    a.total_elements < ((int64_t)1 << 40);
   const unsigned head = fast ? (unsigned)(((16u - (reinterpret_cast<uintptr_t>(a.b.data) & 15u)) & 15u) >> 2) : 0u;
   // max - min a power of two (exact reciprocal): the division in the bin formula can be a multiply
   int exp2 = 0;
@@ -418,7 +420,7 @@ int prepare_histc(const hf_histc_args &a, Prepared &p) {
   const bool pow2 = std::frexp(range, &exp2) == 0.5f && exp2 > -100 && exp2 < 100;
   p.hint = (fast ? HINT_HIST_VEC4 : HINT_GENERIC) | (pow2 ? HINT_HIST_POW2 : 0) | (head << HINT_HIST_HEAD_SHIFT) |
            (global_bins ? HINT_HIST_GLOBAL : 0);
-  p.lds = global_bins ? 0u : (unsigned)a.nbins * 4u;
+  p.lds = global_bins ? 0u : HistcBody::lds_bytes((unsigned)a.nbins);
   p.items = fast ? (unsigned long long)(a.total_elements + 3) / 4 : (unsigned long long)a.total_elements;
   return HF_OK;
 }
@@ -505,15 +507,16 @@ unsigned long long wanted_blocks(const Prepared &p, unsigned threads) {
 // Default grid of one kernel inside a block of `block_threads` threads: enough workgroups
 // to fill every CU sixteen times over, never more than the work asks for.  The streaming
 // bodies stride over the rest; a larger grid evens out their tail.  The histogram is the
-// exception: every block flushes its LDS bins with one global atomic per bin, so it runs
-// one block per CU and keeps eight loads per lane in flight instead.
+// exception: every block flushes its LDS bins with one global atomic per bin, and its input
+// stream runs fastest with about twelve wavefronts per CU (four 16-byte loads in flight per lane:
+// 48 KB per CU; twice that is slower), so it gets as many blocks per CU as make up twelve
+// wavefronts, within what fits next to each other.
 unsigned default_grid(const Prepared &p, unsigned own_threads, unsigned block_threads) {
   const unsigned long long want = wanted_blocks(p, own_threads);
   const unsigned per_cu = std::max(1u, 2048u / block_threads);
-  // (two per CU when it shares its blocks with a partner that ends early)
-  const unsigned long long cap = p.id == K_HISTC
-                                     ? (unsigned long long)cu_count() * (own_threads == block_threads ? 1u : 2u)
-                                     : (unsigned long long)cu_count() * per_cu * 16ull;
+  const unsigned hist_per_cu = std::min(per_cu, std::max(1u, 768u / own_threads));
+  const unsigned long long cap = p.id == K_HISTC ? (unsigned long long)cu_count() * hist_per_cu
+                                                 : (unsigned long long)cu_count() * per_cu * 16ull;
   return (unsigned)std::min(std::max(want, 1ull), cap);
 }
 
@@ -611,7 +614,7 @@ int pair_call_only(const hf_plan *plan) {
 extern "C" {
 
 HF_API const char *hf_last_error(void) { return g_error.c_str(); }
-HF_API int hf_version(void) { return 200; }
+HF_API int hf_version(void) { return 300; }
 
 HF_API int hf_config_load_text(const char *fusion_yaml, const char *kernels_yaml, hf_config **out) try {
   if (!out) return fail(HF_EINVAL, "null output pointer");
@@ -714,11 +717,14 @@ HF_API int hf_plan_create(const hf_config *cfg, int fusion_index, const char *pr
   *out = nullptr;
   if (!cfg || !preset) return fail(HF_EINVAL, "null argument");
   if (fusion_index < 0 || fusion_index >= (int)cfg->cfg.fusions.size()) return fail(HF_EINVAL, "fusion index out of range");
-  const Preset *p = find_preset(preset);
-  if (!p) return fail(HF_ENOTFOUND, std::string("unknown preset '") + preset + "' (vfuse_lb, vfuse, hfuse, hfuse_lb)");
+  const FusionRow &f = cfg->cfg.fusions[fusion_index];
+  // "shipped": the preset the entry names with its `Preset:` key, the thread partition without one
+  const std::string entry_preset = f.preset.empty() ? "hfuse" : f.preset;
+  const std::string asked = std::strcmp(preset, "shipped") == 0 ? entry_preset : std::string(preset);
+  const Preset *p = find_preset(asked);
+  if (!p) return fail(HF_ENOTFOUND, std::string("unknown preset '") + preset + "' (vfuse_lb, vfuse, hfuse, hfuse_lb, or shipped)");
   if (split_threads > 0 && split_threads % (int)kWave != 0)
     return fail(HF_EINVAL, "split_threads must be a multiple of the 64-lane wavefront");
-  const FusionRow &f = cfg->cfg.fusions[fusion_index];
   if (f.kernels.size() != 2 && f.kernels.size() != 3) return unsupported_size(f);
   std::unique_ptr<hf_plan> plan(new hf_plan());  // freed on every early return and on an exception
   plan->preset = p;
@@ -790,6 +796,17 @@ HF_API int hf_plan_create(const hf_config *cfg, int fusion_index, const char *pr
       return rc;
     }
   }
+  if (split_idx == HF_SPLIT_TABLE && split_threads <= 0 && p->base_line && f.blocks.size() == 2) {
+    // the pair's tuned vertical shape: `Blocks` threads run each body, both from thread 0
+    rc = hf_plan_set_block(plan.get(), (int)f.blocks[0], (int)f.blocks[1]);
+    if (rc != HF_OK) {
+      return rc;
+    }
+  }
+  if (split_idx == HF_SPLIT_TABLE && split_threads <= 0 && asked == entry_preset) {
+    plan->grid_override[0] = f.grids[0];   // `Grids:` belongs to the entry's own preset
+    plan->grid_override[1] = f.grids[1];
+  }
   if (is_crypto(plan->ids[0]) && !p->base_line && plan->part.launch_threads > 512) {
     return fail(HF_EINVAL, "search kernels are built for fused blocks of at most 512 threads");
   }
@@ -852,7 +869,7 @@ HF_API int hf_plan_set_grids(hf_plan *plan, int grid1, int grid2) try {
 HF_API int hf_plan_set_block(hf_plan *plan, int threads1, int threads2) try {
   if (!plan) return fail(HF_EINVAL, "null plan");
   if (int prc = pair_call_only(plan)) return prc;
-  if (plan->preset->base_line) return fail(HF_EINVAL, "vertical presets have no thread partition to set");
+  // (under a vertical preset both bodies start at thread 0: the two counts are the threads that run each body)
   if (threads1 <= 0 || threads2 <= 0 || threads1 % (int)kWave || threads2 % (int)kWave)
     return fail(HF_EINVAL, "both parts must be positive multiples of the 64-lane wavefront");
   // Same rule as the re-split of the reference's Context (KernelFusion.h:72): BlockDim.X = threads / BlockDim.Y.
@@ -863,7 +880,7 @@ HF_API int hf_plan_set_block(hf_plan *plan, int threads1, int threads2) try {
       return fail(HF_EINVAL, "thread count does not divide by BlockDim.Y of '" + rows[i].name + "'");
     rows[i].block_dim.x = (uint32_t)want[i] / rows[i].block_dim.y;
   }
-  if (is_crypto(plan->ids[0]) && threads1 + threads2 > 512)
+  if (is_crypto(plan->ids[0]) && (plan->preset->base_line ? std::max(threads1, threads2) : threads1 + threads2) > 512)
     return fail(HF_EINVAL, "search kernels are built for fused blocks of at most 512 threads");
   Partition part;
   std::string err;
@@ -1197,6 +1214,9 @@ int do_launch_fused(const hf_plan *plan, const Prepared &p1, const Prepared &p2,
     const unsigned block = std::max(g.d1, g.d2);
     g.grid1 = p1.exact_grid ? exact : (grid_blocks > 0 ? (unsigned)grid_blocks : default_grid(p1, g.d1, block));
     g.grid2 = p2.exact_grid ? exact : (grid_blocks > 0 ? (unsigned)grid_blocks : default_grid(p2, g.d2, block));
+    // hf_plan_set_grids / the entry's `Grids:`: a few resident blocks whose threads stride over each body's work in turn
+    if (grid_blocks <= 0 && plan->grid_override[0] && !p1.exact_grid) g.grid1 = plan->grid_override[0];
+    if (grid_blocks <= 0 && plan->grid_override[1] && !p2.exact_grid) g.grid2 = plan->grid_override[1];
     const size_t lds = 4 * kBarrierWords + g.lds1 + g.lds2;
     const unsigned grid = std::max(g.grid1, g.grid2);
     if (!counters_fit(grid, block)) return fail(HF_EINVAL, kCounterMsg);

@@ -31,6 +31,10 @@ typedef unsigned int u32x2 __attribute__((ext_vector_type(2)));
 
 enum { BAR_WORKGROUP = 0, BAR_SUBSET = 1 };
 
+#ifndef HF_SYNC_BACKOFF
+#define HF_SYNC_BACKOFF 1  // 0: a parked wave polls its arrival counter every 64 cycles (experiment switch)
+#endif
+
 enum KernelId {
   K_IM2COL = 0,
   K_MAXPOOL,
@@ -77,6 +81,7 @@ struct SubBlock {
   unsigned phase;     // barriers this thread has passed
   unsigned gbase;     // index of this half's thread 0 among all threads that run this kernel
   unsigned gthreads;  // number of threads that run this kernel in the whole launch
+  bool whole = false; // BAR_SUBSET only: this body runs on every wave of the workgroup, so the hardware barrier serves it
 
   // Flat work-item index and stride of a body that walks a 1-D range.  Equal to
   // bid * nthreads + tid and nblocks * nthreads except where a block lends the idle
@@ -92,14 +97,26 @@ struct SubBlock {
     if constexpr (BAR == BAR_WORKGROUP) {
       __syncthreads();
     } else {
+      if (whole) {  // wave-uniform: every wave of the workgroup runs this body and reaches this barrier
+        __syncthreads();
+        return;
+      }
       phase++;
       // Release this wave's LDS/global writes to the workgroup, arrive, wait, acquire.
       __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
       if (lane() == 0) {
         __hip_atomic_fetch_add(bar, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
         const unsigned target = phase * nwaves();
-        while (__hip_atomic_load(bar, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP) < target)
-          __builtin_amdgcn_s_sleep(1);
+        // A parked wave polls the LDS its working siblings add into: the naps grow (64, 128, 256, then 512
+        // cycles) so that a long wait costs a handful of LDS reads instead of one every 64 cycles.
+        unsigned polls = 0;
+        while (__hip_atomic_load(bar, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP) < target) {
+          if (!HF_SYNC_BACKOFF || polls < 2) __builtin_amdgcn_s_sleep(1);
+          else if (polls < 4) __builtin_amdgcn_s_sleep(2);
+          else if (polls < 8) __builtin_amdgcn_s_sleep(4);
+          else __builtin_amdgcn_s_sleep(8);
+          polls++;
+        }
       }
       __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup");
     }
@@ -264,12 +281,13 @@ __device__ __forceinline__ void vertical_block(const typename K1::Args &a1, cons
   constexpr int B1 = K1::kBarriers ? BAR_SUBSET : BAR_WORKGROUP;
   constexpr int B2 = K2::kBarriers ? BAR_SUBSET : BAR_WORKGROUP;
   const unsigned wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  // A body as wide as the block runs on every wave, so its barriers are the workgroup's own.
   if (wave < (g.d1 >> 6) && bid < g.grid1) {
-    SubBlock<B1> sb{tid, g.d1, bid, g.grid1, bars + 0, 0, bid * g.d1, g.grid1 * g.d1};
+    SubBlock<B1> sb{tid, g.d1, bid, g.grid1, bars + 0, 0, bid * g.d1, g.grid1 * g.d1, g.d1 == blockDim.x};
     K1::run(a1, sb, smem + 4 * kBarrierWords, g.hint1);
   }
   if (wave < (g.d2 >> 6) && bid < g.grid2) {
-    SubBlock<B2> sb{tid, g.d2, bid, g.grid2, bars + 1, 0, bid * g.d2, g.grid2 * g.d2};
+    SubBlock<B2> sb{tid, g.d2, bid, g.grid2, bars + 1, 0, bid * g.d2, g.grid2 * g.d2, g.d2 == blockDim.x};
     K2::run(a2, sb, smem + 4 * kBarrierWords + g.lds1, g.hint2);
   }
 }

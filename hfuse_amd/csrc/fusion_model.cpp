@@ -191,9 +191,10 @@ bool parse_config(const char *fusion_yaml, const char *kernels_yaml, Config &cfg
         }
       }
       if (const YamlNode *bl = n.get("Blocks")) {
-        // not in the reference's schema: the block shape of a three-kernel entry, one thread count per kernel
-        if (bl->kind != YamlNode::Seq || bl->seq.size() != ks->seq.size() || ks->seq.size() != 3) {
-          err = "fusion list: " + at(*bl) + "'Blocks' must list one thread count per kernel of a three-kernel entry";
+        // not in the reference's schema: one thread count per kernel -- the block shape of a three-kernel entry, or
+        // of a pair under a vertical preset
+        if (bl->kind != YamlNode::Seq || bl->seq.size() != ks->seq.size() || (ks->seq.size() != 3 && ks->seq.size() != 2)) {
+          err = "fusion list: " + at(*bl) + "'Blocks' must list one thread count per kernel of a pair or a three-kernel entry";
           return false;
         }
         for (auto &b : bl->seq) {
@@ -205,9 +206,28 @@ bool parse_config(const char *fusion_yaml, const char *kernels_yaml, Config &cfg
           f.blocks.push_back(t);
         }
       }
+      if (const YamlNode *pr = n.get("Preset")) {
+        // not in the reference's schema: which of the driver's four presets (main.cpp:182-193) this entry ships with
+        if (pr->kind != YamlNode::Scalar || !find_preset(pr->scalar)) {
+          err = "fusion list: " + at(*pr) + "'Preset' must be one of vfuse_lb, vfuse, hfuse, hfuse_lb";
+          return false;
+        }
+        f.preset = pr->scalar;
+      }
+      if (const YamlNode *gr = n.get("Grids")) {
+        uint32_t g0 = 0, g1 = 0;
+        if (gr->kind != YamlNode::Seq || gr->seq.size() != 2 || ks->seq.size() != 2 || !to_uint(&gr->seq[0], g0) ||
+            !to_uint(&gr->seq[1], g1) || g0 > (1u << 24) || g1 > (1u << 24)) {
+          err = "fusion list: " + at(*gr) + "'Grids' must list two workgroup counts (0 = the library's) of a pair";
+          return false;
+        }
+        f.grids[0] = g0;
+        f.grids[1] = g1;
+      }
       for (auto &kv : n.map)
         if (kv.first != "File" && kv.first != "Kernels" && kv.first != "Split" && kv.first != "Threads" &&
-            kv.first != "Lending" && kv.first != "Barrier" && kv.first != "LaunchBound" && kv.first != "Blocks") {
+            kv.first != "Lending" && kv.first != "Barrier" && kv.first != "LaunchBound" && kv.first != "Blocks" &&
+            kv.first != "Preset" && kv.first != "Grids") {
           err = "fusion list: " + at(kv.second) + "unknown key '" + kv.first + "'";
           return false;
         }

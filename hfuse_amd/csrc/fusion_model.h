@@ -35,7 +35,10 @@ struct FusionRow {
   int lending = -1;      // optional `Lending:` key: 0 / 1 switch wave lending off / on, -1 = library default
   int launch_bound = -1; // optional `LaunchBound:` key: 0 / 1 pick the plain / register-bounded build, -1 = the preset's
   int barrier = -1;      // optional `Barrier:` key: an HF_BARRIER_* mode, -1 = library default
-  std::vector<uint32_t> blocks;  // optional `Blocks:` key of a three-kernel entry: threads of each kernel in the fused block
+  std::vector<uint32_t> blocks;  // optional `Blocks:` key: threads of each kernel -- the block shape of a three-kernel entry,
+                                 // or of a pair under a vertical preset (both bodies start at thread 0)
+  std::string preset;            // optional `Preset:` key: the preset this entry ships with ("" = hfuse)
+  uint32_t grids[2] = {0, 0};    // optional `Grids:` key of a pair: workgroups each kernel strides over under `Preset` (0 = the library's)
 };
 
 struct Config {

@@ -180,8 +180,12 @@ class Plan:
         return f.value, b.value
 
     def bind_constants(self, constants: Optional["Constants"]) -> None:
-        """Fused launches of this plan use a copy of `constants` instead of the process-wide set (None unbinds)."""
+        """Fused launches of this plan use a copy of `constants` instead of the process-wide set (None unbinds).
+
+        The copy is a snapshot taken now (later changes of `constants` do not reach the plan) and holds the raw
+        device pointer of the Ethash DAG, so the plan keeps `constants` -- and through it the DAG tensor -- alive."""
         check(L.lib().hf_plan_bind_constants(self._h, constants._h if constants is not None else None))
+        self._consts = constants
 
     def local_index(self, half: int, tid: int):
         out = L.Dim3()

@@ -254,8 +254,16 @@ def test_set_block_rules():
     for bad in ((100, 256), (0, 256), (128, 0), (512, 768), (128, 64 * 3 + 8)):
         with pytest.raises(hfuse_amd.HfuseError):
             plan.set_block(*bad)
-    with pytest.raises(hfuse_amd.HfuseError):
-        cfg.plan(1, "vfuse").set_block(128, 128)
+    # under a vertical preset both bodies start at thread 0 (KernelFusion.h:76-78): the two counts are the threads
+    # that run each body, the block is the larger of them
+    v = cfg.plan(1, "vfuse")
+    v.set_block(128, 512)
+    q = v.partition
+    assert (list(q.lo), list(q.hi), q.launch_threads) == ([0, 0], [128, 512], 512)
+    assert q.name.decode().endswith("_fused_kernel_vfuse_block_128_512")
+    for bad in ((100, 256), (128, 1088)):
+        with pytest.raises(hfuse_amd.HfuseError):
+            v.set_block(*bad)
     plan.set_grids(3, 5)
     plan.set_lending(False)
     with pytest.raises(hfuse_amd.HfuseError):
@@ -695,9 +703,34 @@ def test_three_kernel_plans_refuse_the_calls_that_shape_a_pair():
     # the shipped three-kernel list and its Blocks key
     t = hfuse_amd.triples_config()
     assert [list(t.plan(i).partition_n.hi)[:3] for i in range(3)] == [[64, 192, 256], [256, 640, 768], [512, 768, 1024]]
-    with pytest.raises(hfuse_amd.HfuseError) as e:
-        Config("- File: t\n  Kernels:\n    - a\n    - b\n  Blocks:\n    - 64\n    - 64\n", KERNELS_MAP.replace("im2col_kernel:", "a:").replace("MaxPoolForward:", "b:"))
+    with pytest.raises(hfuse_amd.HfuseError) as e:   # one thread count per kernel
+        Config("- File: t\n  Kernels:\n    - a\n    - b\n  Blocks:\n    - 64\n    - 64\n    - 64\n", KERNELS_MAP.replace("im2col_kernel:", "a:").replace("MaxPoolForward:", "b:"))
     assert e.value.code == L.HF_EPARSE and "Blocks" in e.value.message
+
+
+def test_shipped_preset_and_its_keys():
+    """`Preset:` names the preset an entry ships with (one of the driver's four, main.cpp:182-193); "shipped" asks for
+    it.  Under a vertical preset `Blocks:` gives the threads that run each body and `Grids:` the workgroups each
+    body strides over; a plan of any other preset ignores both."""
+    text = ("- File: a\n  Kernels:\n    - im2col_kernel\n    - MaxPoolForward\n  Split: 256\n  Threads: 704\n"
+            "  Preset: vfuse\n  Blocks:\n    - 768\n    - 1024\n  Grids:\n    - 256\n    - 512\n"
+            "- File: b\n  Kernels:\n    - im2col_kernel\n    - MaxPoolForward\n  Split: 256\n  Threads: 704\n")
+    cfg = Config(text, KERNELS_MAP)
+    v = cfg.plan(0, "shipped").partition
+    assert v.name.decode() == "im2col_kernel_MaxPoolForward_fused_kernel_vfuse_block_768_1024"
+    assert (list(v.lo), list(v.hi), v.launch_threads) == ([0, 0], [768, 1024], 1024)
+    h = cfg.plan(0, "hfuse").partition                      # the thread partition keeps its own tuned shape
+    assert (list(h.hi), h.launch_threads) == ([256, 704], 704)
+    assert cfg.plan(0, "vfuse", 0).partition.launch_threads == 512   # an explicit variant: the table's BlockDims
+    s = cfg.plan(1, "shipped").partition                    # no Preset key: the thread partition
+    assert s.name.decode().startswith("im2col_kernel_MaxPoolForward_fused_kernel_hfuse") and list(s.hi) == [256, 704]
+    for bad in ("  Preset: fast\n", "  Grids:\n    - 1\n", "  Grids: 5\n", "  Blocks:\n    - 100\n    - 64\n"):
+        with pytest.raises(hfuse_amd.HfuseError) as e:
+            Config("- File: a\n" + bad + "  Kernels:\n    - im2col_kernel\n    - MaxPoolForward\n", KERNELS_MAP)
+        assert e.value.code == L.HF_EPARSE
+    with pytest.raises(hfuse_amd.HfuseError) as e:
+        cfg.plan(0, "fastest")
+    assert e.value.code == L.HF_ENOTFOUND
 
 
 def test_header_symbols_are_all_exported():
@@ -710,7 +743,7 @@ def test_header_symbols_are_all_exported():
     lib = L.lib()
     for name in declared:
         assert hasattr(lib, name), name
-    assert lib.hf_version() >= 100
+    assert lib.hf_version() == L.ABI_VERSION == 300   # _lib.lib() refuses any other build
 
 
 def test_deep_nesting_is_refused_not_followed():
