@@ -50,11 +50,16 @@ TRAFFIC_BYTES = {"bn_upsample": 156.54e6, "im2col_maxpool": 443.27e6, "histc_max
 OPS_SHA256D = 4336
 OPS_BLAKE2B = 2528
 ETHASH_BYTES = 8192               # 64 accesses x 128 bytes of DAG per hash
+# VALU instructions a wavefront issues per hash (SQ_INSTS_VALU of the native kernels over 2^24 hashes, x 64 lanes / 2^24:
+# profiles/all_pairs_sq_counters.md) and the rate one CU issues them at: 64 lanes per clock
+VALU_INSTS_SHA256D = 3082
+VALU_INSTS_BLAKE2B = 1101
+VALU_ISSUE_GLANES = 256 * 64 * 2.4  # 256 CUs x 64 lanes x 2.4 GHz, in G lane-instructions/s
 
-# What a fused tensor pair could reach at best: its bytes at the rates bare loops reach on this part (16-byte
-# non-temporal accesses over 512 MiB: reads 7.1 TB/s, writes 6.5 TB/s), reads and writes after each other with no
-# turnaround cost, plus the 1.7 us an empty kernel takes.  (read bytes, written bytes) of both kernels of a pair:
-READ_GBPS_MEASURED, WRITE_GBPS_MEASURED, EMPTY_LAUNCH_US = 7100.0, 6500.0, 1.7
+# What a fused tensor pair could reach at best: its bytes at the rates the library's bare stream kernels reach on
+# this part in this run (hfuse_amd.streams: contiguous 16-byte non-temporal reads and writes over rotating 512 MiB
+# buffers), reads and writes after each other with no turnaround cost, plus the time an empty kernel takes.
+# (read bytes, written bytes) of both kernels of a pair:
 PAIR_READ_WRITE_BYTES = {
     "im2col_maxpool": (4 * 32 * 64 * (56 * 56 + 112 * 112), 4 * 32 * 576 * 3136 + 12 * 32 * 64 * 56 * 56),
     "bn_upsample": (4 * 32 * 256 * 28 * 28 + 4 * 32 * 64 * 56 * 56, 2 * 4 * 256 + 4 * 32 * 64 * 112 * 112),
@@ -91,6 +96,11 @@ def parse():
                     help="full rotations of a tensor pair's buffer sets per timing sample (launch floor, independent of --steps)")
     ap.add_argument("--calibrate-copy", type=int, default=0, metavar="MIB",
                     help="also run the plain copy kernel on MIB mebibytes (the unit HBM counters are scaled by)")
+    ap.add_argument("--calibrate-streams", dest="streams", action="store_true", default=True,
+                    help="measure the stream ceilings (contiguous reads / writes, random 128-byte lines, 1 : 4 copy, empty "
+                         "launch) with the library's bare stream kernels in this run; they feed `streaming_bound` (default)")
+    ap.add_argument("--no-streams", dest="streams", action="store_false", help="skip the stream ceilings")
+    ap.add_argument("--search-samples", type=int, default=5, help="interleaved samples per mode of a search pair")
     return ap.parse_args()
 
 
@@ -100,7 +110,7 @@ from hfuse_amd.workloads import (SEED, BENCH_TENSOR_PAIRS, TENSOR_KERNELS, Searc
 
 def candidate_plans(cfg, k1, k2, sweep):
     i = cfg.find_fusion(k1, k2)
-    out = [("table", cfg.plan(i))]
+    out = [("table", cfg.plan(i, "shipped"))]
     if sweep:
         for idx in range(cfg.num_splits(i)):
             try:
@@ -119,56 +129,90 @@ def blockidx_plan(cfg, i):
     return plan
 
 
+def spread(samples):
+    """{mode: [min, median, max]} of the per-launch milliseconds of every mode."""
+    return {k: [min(v), statistics.median(v), max(v)] for k, v in samples.items()}
+
+
+def shipped_mode(plan):
+    """Name of the form a plan runs in: one of the keys `judge` compares."""
+    part = plan.partition
+    name = part.name.decode()
+    if "_fused_kernel_vfuse" in name:
+        return "vfuse"
+    if part.barrier_mode == 3:          # HF_BARRIER_BLOCKIDX
+        return "blockidx"
+    return "hfuse_lb" if plan.launch_waves[1] else "hfuse"
+
+
 def judge(res):
-    """Adds speedup, the fastest way to run the pair and horizontal-vs-vertical to a per-pair result."""
+    """Adds speedup, the fastest way to run the pair and horizontal-vs-vertical to a per-pair result.  `t_fused_ms`
+    is the form the fusion list ships for the pair; `t_hfuse_ms` its thread partition, `t_vfuse_ms` its vertical kernel."""
     res["speedup_pct"] = (res["t_b2b_ms"] / res["t_fused_ms"] - 1.0) * 100.0
     ways = {"back_to_back": res["t_b2b_ms"], "two_streams": res["t_two_streams_ms"], "vfuse": res["t_vfuse_ms"],
-            "hfuse": res["t_fused_ms"], "hfuse_lb": res["t_fused_lb_ms"]}
+            "hfuse": res["t_hfuse_ms"], "hfuse_lb": res["t_fused_lb_ms"]}
     if "t_blockidx_ms" in res:
         ways["blockidx"] = res["t_blockidx_ms"]
     res["best_mode"] = min(ways, key=ways.get)
-    res["hfuse_vs_vfuse_pct"] = (res["t_vfuse_ms"] / res["t_fused_ms"] - 1.0) * 100.0
-    res["hfuse_vs_two_streams_pct"] = (res["t_two_streams_ms"] / res["t_fused_ms"] - 1.0) * 100.0
+    # modes within 0.3 % of the fastest run at the same speed for every practical purpose
+    res["modes_within_0p3pct_of_best"] = sorted(k for k, v in ways.items() if v <= ways[res["best_mode"]] * 1.003)
+    res["hfuse_vs_vfuse_pct"] = (res["t_vfuse_ms"] / res["t_hfuse_ms"] - 1.0) * 100.0
+    res["hfuse_vs_two_streams_pct"] = (res["t_two_streams_ms"] / res["t_hfuse_ms"] - 1.0) * 100.0
+    res["hfuse_speedup_pct"] = (res["t_b2b_ms"] / res["t_hfuse_ms"] - 1.0) * 100.0
 
 
 # ------------------------------------------------------------------ tensor pairs
 def time_tensor_pair(cfg, pair, rotations, sweep, fused_only, rounds=5):
-    """-> dict with per-launch milliseconds of native A, native B, back to back, two streams, the vertical
-    baseline, the fused kernel and its register-bounded build.
+    """-> dict with per-launch milliseconds of native A, native B, back to back, two streams, the form the fusion list
+    ships for the pair (`t_fused_ms`), its thread partition, its vertical kernel, the block-index partition and the
+    register-bounded build.
 
     Every sample is `rotations` full cycles through the pair's buffer sets (whatever --steps says), each
     call continues the rotation where the previous one stopped, and the modes are interleaved in
-    `rounds` rounds whose median is reported, so slow drifts of the clocks hit all modes alike."""
+    `rounds` rounds whose median is reported (minimum and maximum next to it), so slow drifts of the clocks hit all
+    modes alike."""
     i = cfg.find_fusion(pair.k1, pair.k2)
-    plans = candidate_plans(cfg, pair.k1, pair.k2, sweep)
     nsets = len(pair.sets)
     per = max(1, rotations) * nsets
-    plan, label = plans[0][1], plans[0][0]
-    if len(plans) > 1:
+    shipped = cfg.plan(i, "shipped")
+    mode = shipped_mode(shipped)
+    plan, label = shipped, "table"
+    if sweep:
         best = None
-        for lab, p in plans:
+        for lab, p in candidate_plans(cfg, pair.k1, pair.k2, sweep):
             t = pair.time(p, 3, 3, per) / per
             if best is None or t < best[0]:
                 best = (t, lab, p)
         _, label, plan = best
     runs = [("t_fused_ms", plan, 3)]
+    alias = {}
     if not fused_only:
         runs = [("t_a_ms", plan, 0), ("t_b_ms", plan, 1), ("t_b2b_ms", plan, 2), ("t_fused_ms", plan, 3),
-                ("t_two_streams_ms", plan, 4),                     # the launch pattern of the reference's own traces
-                ("t_vfuse_ms", cfg.plan(i, "vfuse"), 3),           # the reference's vertical baseline
-                ("t_fused_lb_ms", cfg.plan(i, "hfuse_lb"), 3),     # the same block shape, register-bounded build
-                ("t_blockidx_ms", blockidx_plan(cfg, i), 3)]       # each workgroup runs one of the two kernels
+                ("t_two_streams_ms", plan, 4)]                     # the launch pattern of the reference's own traces
+        others = [("t_hfuse_ms", "hfuse", lambda: cfg.plan(i, "hfuse")),          # the thread partition at its tuned shape
+                  ("t_vfuse_ms", "vfuse", lambda: cfg.plan(i, "vfuse")),          # the reference's vertical baseline
+                  ("t_blockidx_ms", "blockidx", lambda: blockidx_plan(cfg, i))]   # each workgroup runs one of the two kernels
+        for key, m, make in others:
+            if m == mode and not sweep:
+                alias[key] = "t_fused_ms"       # the shipped form: one plan, one set of samples
+            else:
+                runs.append((key, make(), 3))
+        runs.append(("t_fused_lb_ms", cfg.plan(i, "hfuse_lb"), 3))  # the thread partition's register-bounded build
     for _, p, m in runs:                                            # one untimed rotation per mode
         pair.time(p, m, 0, nsets)
     samples = {k: [] for k, _, _ in runs}
     for _ in range(rounds):
         for key, p, m in runs:
             samples[key].append(pair.time(p, m, 2, per) / per)
+    for key, src in alias.items():
+        samples[key] = samples[src]
     res = {k: statistics.median(v) for k, v in samples.items()}
+    res["min_median_max_ms"] = spread(samples)
     res["launches_per_sample"], res["rounds"], res["buffer_sets"] = per, rounds, nsets
     if not fused_only:
-        res["lb_waves_per_simd"] = runs[6][1].launch_waves[1]
+        res["lb_waves_per_simd"] = runs[-1][1].launch_waves[1]
     res["split"] = label
+    res["shipped_mode"] = mode
     part = plan.partition
     res["fused_name"] = part.name.decode()
     res["threads"] = [part.hi[0] - part.lo[0], part.hi[1] - part.lo[1]]
@@ -229,7 +273,7 @@ def sia_digest(header80: bytes, nonce: int) -> bytes:
     return hashlib.blake2b(msg, digest_size=32).digest()
 
 
-def run_search_pair(cfg, name, log2_a, log2_b, sweep, fused_only, steps=0, warmup=0, iters=2):
+def run_search_pair(cfg, name, log2_a, log2_b, sweep, fused_only, steps=0, warmup=0, iters=5):
     """sha256d+blake2b or ethash+blake2b over 2^log2_a + 2^log2_b nonces.  With steps > 0 the fused
     kernel is also run for the contract's timed region: `warmup` untimed launches, then exactly
     `steps` launches between two synchronisations."""
@@ -267,18 +311,36 @@ def run_search_pair(cfg, name, log2_a, log2_b, sweep, fused_only, steps=0, warmu
             best = (t, label, plan)
     _, label, plan = best
     fused_grid = grid_of(plan)
+    mode = shipped_mode(plan)
+    alias = {}
     if not fused_only:
-        vplan, lbplan = bound(cfg.plan(i, "vfuse")), bound(cfg.plan(i, "hfuse_lb"))
+        lbplan = bound(cfg.plan(i, "hfuse_lb"))
         runs = [("t_a_ms", base, 0, grid), ("t_b_ms", base, 1, 0), ("t_b2b_ms", base, 2, grid),
-                ("t_fused_ms", plan, 3, fused_grid), ("t_two_streams_ms", base, 4, grid),
-                ("t_vfuse_ms", vplan, 3, grid), ("t_fused_lb_ms", lbplan, 3, grid_of(lbplan))]
+                ("t_fused_ms", plan, 3, fused_grid), ("t_two_streams_ms", base, 4, grid)]
+
+        # (in every form Ethash scans grid * its own threads nonces: grid_of keeps its range at `na`)
+        others = [("t_hfuse_ms", "hfuse", lambda: bound(cfg.plan(i, "hfuse"))),
+                  ("t_vfuse_ms", "vfuse", lambda: bound(cfg.plan(i, "vfuse"))),
+                  ("t_blockidx_ms", "blockidx", lambda: bound(blockidx_plan(cfg, i)))]
+        for key, m, make in others:
+            if m == mode and not sweep:
+                alias[key] = "t_fused_ms"
+            else:
+                p_ = make()
+                runs.append((key, p_, 3, grid_of(p_)))
+        runs.append(("t_fused_lb_ms", lbplan, 3, grid_of(lbplan)))
     else:
         runs = [("t_fused_ms", plan, 3, fused_grid)]
     samples = {k: [] for k, _, _, _ in runs}
-    for _ in range(iters):                       # modes interleaved, one launch per sample
+    for _ in range(max(1, iters)):               # modes interleaved, one launch per sample
         for key, p, m, g in runs:
             samples[key].append(p.time(m, [a1], [a2], 0, 1, g))
+    for key, src in alias.items():
+        samples[key] = samples[src]
     res.update({k: statistics.median(v) for k, v in samples.items()})
+    res["min_median_max_ms"] = spread(samples)
+    res["samples_per_mode"] = max(1, iters)
+    res["shipped_mode"] = mode
     if not fused_only:
         res["lb_waves_per_simd"] = lbplan.launch_waves[1]
     if steps > 0:
@@ -323,7 +385,7 @@ def run_search_pair(cfg, name, log2_a, log2_b, sweep, fused_only, steps=0, warmu
     ea, eb = H.new_search_results(), H.new_search_results()
     e1 = H.ethash_args(ea, 0) if ethash else H.sha256d_args(ea, na, 0)
     e2 = H.blake2b_args(eb, nb, 0, easy_target)
-    eplan = cfg.plan(i)
+    eplan = cfg.plan(i, "shipped")
     eplan.bind_constants(easy)
     eplan.launch(e1, e2, grid_blocks=fused_grid)
     na2, nb2 = H.new_search_results(), H.new_search_results()
@@ -502,6 +564,11 @@ def main():
             H.copy_f32(src[i % 4], dst[i % 4])
         torch.cuda.synchronize()
         del src, dst
+    ceilings = None
+    if args.streams:
+        from hfuse_amd import streams
+        ceilings = streams.measure()
+        torch.cuda.empty_cache()
     all_names = list(TENSOR_NAMES + SEARCH_NAMES)
     names = all_names if args.pairs == "all" else [n for n in args.pairs.split(",") if n]
     if args.headline not in names:
@@ -533,11 +600,15 @@ def main():
             r["a_gbps"] = pair.bytes1 / (r["t_a_ms"] * 1e-3) / 1e9
             r["b_gbps"] = pair.bytes2 / (r["t_b_ms"] * 1e-3) / 1e9
             judge(r)
-            rd, wr = PAIR_READ_WRITE_BYTES[name]
-            floor_ms = (rd / READ_GBPS_MEASURED + wr / WRITE_GBPS_MEASURED) * 1e-6 + EMPTY_LAUNCH_US * 1e-3
-            r["streaming_bound"] = {"fused_floor_ms": floor_ms, "max_speedup_pct": (r["t_b2b_ms"] / floor_ms - 1.0) * 100.0,
-                                    "fused_over_floor": r["t_fused_ms"] / floor_ms,
-                                    "basis": "read bytes at 7.1 TB/s + written bytes at 6.5 TB/s (bare loops on this part) + 1.7 us launch"}
+            if ceilings:
+                rd, wr = PAIR_READ_WRITE_BYTES[name]
+                floor_ms = (rd / ceilings["read_gbps"] + wr / ceilings["write_gbps"]) * 1e-6 + ceilings["empty_launch_us"] * 1e-3
+                r["streaming_bound"] = {"fused_floor_ms": floor_ms, "max_speedup_pct": (r["t_b2b_ms"] / floor_ms - 1.0) * 100.0,
+                                        "fused_over_floor": r["t_fused_ms"] / floor_ms,
+                                        "read_gbps": ceilings["read_gbps"], "write_gbps": ceilings["write_gbps"],
+                                        "empty_launch_us": ceilings["empty_launch_us"],
+                                        "basis": "read bytes at read_gbps + written bytes at write_gbps (the library's bare stream "
+                                                 "kernels, measured in this run) + one empty launch"}
         if name == args.headline:
             r["wall_ms_per_step"], r["event_ms_per_step"] = timed_region(plan, pair)
         r["check"] = check_tensor_pair(name, pair, plan)
@@ -550,7 +621,7 @@ def main():
         lb = args.search_log2 + 2 if (args.search_log2 and name == "ethash_blake2b") else (args.search_log2 or 30)
         head = name == args.headline
         r = run_search_pair(cfg, name, la, lb, sweep, args.fused_only, steps=args.steps if head else 0,
-                            warmup=args.warmup if head else 0)
+                            warmup=args.warmup if head else 0, iters=args.search_samples)
         r["log2_nonces"] = [la, lb]
         na, nb = r["nonces"]
         tf = r["t_fused_ms"] * 1e-3
@@ -560,14 +631,21 @@ def main():
             r["fused_valu_gops"] = ops / tf / 1e9
             r["roofline_frac"] = r["fused_valu_gops"] / VALU_PEAK_GOPS
             r["roofline_bound"] = "valu_int32"
+            # the same against the rate a CU issues VALU instructions at (64 lanes a clock): instructions per hash
+            # from the SQ counters x hashes per second
+            r["valu_issue_frac"] = (na * VALU_INSTS_SHA256D + nb * VALU_INSTS_BLAKE2B) / tf / 1e9 / VALU_ISSUE_GLANES
         else:
             r["dag_gbps"] = na * ETHASH_BYTES / tf / 1e9
             r["roofline_frac"] = r["dag_gbps"] / HBM_PEAK_GBPS
             r["roofline_bound"] = "hbm"
             r["blake2b_valu_frac"] = nb * OPS_BLAKE2B / tf / 1e9 / VALU_PEAK_GOPS
+            r["blake2b_valu_issue_frac"] = nb * VALU_INSTS_BLAKE2B / tf / 1e9 / VALU_ISSUE_GLANES
         if not args.fused_only:
             r["a_mhs"] = na / (r["t_a_ms"] * 1e-3) / 1e6
             r["b_mhs"] = nb / (r["t_b_ms"] * 1e-3) / 1e6
+            if name == "sha256d_blake2b":
+                r["a_valu_issue_frac"] = VALU_INSTS_SHA256D * r["a_mhs"] * 1e-3 / VALU_ISSUE_GLANES
+            r["b_valu_issue_frac"] = VALU_INSTS_BLAKE2B * r["b_mhs"] * 1e-3 / VALU_ISSUE_GLANES
             judge(r)
         report[name] = r
         torch.cuda.empty_cache()
@@ -581,6 +659,7 @@ def main():
                 pair = build_pair(f"{k1}+{k2}", k1, k2)
                 r = time_tensor_pair(cfg, pair, args.rotations, sweep, False)
                 r.pop("plan")
+                r.pop("min_median_max_ms")
                 r["fused_gbps"] = (pair.bytes1 + pair.bytes2) / (r["t_fused_ms"] * 1e-3) / 1e9
                 judge(r)
                 extra[pair.name] = r
@@ -665,6 +744,10 @@ def main():
         "config": {"workload": workload, "fused_kernel": h.get("fused_name"), "split_threads": h.get("threads")},
         "throughput": throughput,
         "pairs_at_least_10pct_faster": n_fast,
+        "pairs_slower_than_back_to_back": sorted(n for n, r in report.items() if r.get("speedup_pct", 0.0) < 0.0),
+        "shipped_is_best_mode": {n: r.get("shipped_mode") in r.get("modes_within_0p3pct_of_best", [r.get("shipped_mode")])
+                                 for n, r in report.items()},
+        "stream_ceilings": ceilings,
         "roofline": roofline,
         "cpu_baseline": cpu,
         "pairs": report,

@@ -9,11 +9,14 @@ import ctypes as C
 import os
 
 _HERE = os.path.dirname(os.path.abspath(__file__))
-LIB_PATH = os.path.join(_HERE, "libhfuse_gfx950.so")
+# HFUSE_LIB names another build of the same library (the timing-only take-apart builds of `make takeapart`)
+LIB_PATH = os.environ.get("HFUSE_LIB") or os.path.join(_HERE, "libhfuse_gfx950.so")
 
 HF_OK, HF_EINVAL, HF_EPARSE, HF_ENOTFOUND, HF_EUNSUPPORTED, HF_EHIP, HF_EIO, HF_ENOMEM = 0, -1, -2, -3, -4, -5, -6, -7
 HF_BARRIER_NONE, HF_BARRIER_MATCHED, HF_BARRIER_SUBSET, HF_BARRIER_BLOCKIDX = 0, 1, 2, 3
 HF_SPLIT_TABLE, HF_SPLIT_EXECTIME = -1, -2
+HF_STREAM_EMPTY, HF_STREAM_READ, HF_STREAM_WRITE, HF_STREAM_READ_LINES, HF_STREAM_COPY_1_4 = 0, 1, 2, 3, 4
+HF_STREAM_WRITE_STRIDED, HF_STREAM_WRITE_XCD = 5, 6
 ABI_VERSION = 300          # what hf_version() of a matching library answers
 HF_MAX_SEARCH_RESULTS = 64
 HF_MAX_TENSORINFO_DIMS = 8
@@ -179,6 +182,9 @@ PROTOTYPES = {
                                C.c_int, C.c_int, C.c_int, C.c_void_p, C.POINTER(C.c_float)]),
     "hf_fill_splitmix64": (C.c_int, [C.c_void_p, C.c_uint64, C.c_uint64, C.c_void_p]),
     "hf_copy_f32": (C.c_int, [C.c_void_p, C.c_void_p, C.c_uint64, C.c_void_p]),
+    "hf_stream_probe": (C.c_int, [C.c_int, C.c_void_p, C.c_void_p, C.c_uint64, C.c_int, C.c_int, C.c_void_p]),
+    "hf_time_stream_probe": (C.c_int, [C.c_int, C.c_void_p, C.c_void_p, C.c_uint64, C.c_uint64, C.c_uint64, C.c_int, C.c_int,
+                                       C.c_int, C.c_int, C.c_int, C.c_void_p, C.POINTER(C.c_float)]),
 }
 
 _lib = None

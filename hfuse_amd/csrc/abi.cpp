@@ -579,8 +579,10 @@ namespace {
 // Waves per SIMD the occupancy formula of the reference's printer asks for with this part's constants:
 // B = min_k(regfile / Reg_k / threads_k) blocks per CU, capped by the resident threads
 // (lib/KernelFuser/KernelPrinter.cpp:44-66), times the block's waves, spread over four SIMDs.
+// Rounded up: B blocks of T threads are B * T / 64 waves, and all of them have to fit (5.5 waves per SIMD need 6).
 int formula_waves(const hf_plan *plan) {
-  const unsigned long long w = (unsigned long long)plan->part.bound_blocks * plan->part.launch_threads / (4ull * kWave);
+  const unsigned long long waves = (unsigned long long)plan->part.bound_blocks * (plan->part.launch_threads / kWave);
+  const unsigned long long w = (waves + 3) / 4;
   return (int)std::min<unsigned long long>(std::max<unsigned long long>(w, 1), (unsigned long long)kBoundedWaves);
 }
 
@@ -588,13 +590,32 @@ int formula_waves(const hf_plan *plan) {
 // The launch-bound presets ask for a bounded build when the formula wants more waves per SIMD than the
 // plain build's launch bound of 1024 threads already guarantees (four).
 int plan_build_waves(const hf_plan *plan) {
-  if (plan->n != 2) return 0;  // three-kernel fusions have the plain build only
+  if (plan->n != 2) return plan->preset->launch_bound ? kBoundedWaves : 0;  // three-kernel fusions: plain, or bounded for 8 waves
   if (!plan->preset->base_line && plan->barrier_mode == HF_BARRIER_BLOCKIDX) return 0;  // no bounded build
   const int formula = formula_waves(plan);
   const bool want = plan->bounded >= 0 ? plan->bounded != 0 : plan->preset->launch_bound && formula > 4;
   if (!want) return 0;
   const int built = built_bound_waves(plan->ids[0], plan->ids[1], plan->bound_waves ? plan->bound_waves : formula);
   return plan->preset->base_line ? kBoundedWaves : built;   // the vertical baseline has the 8-wave build only
+}
+
+// The three-kernel lists that are instantiated, in the order they are built in (the reference's configs/
+// im2col_maxpool_norm.yaml, maxpool_summary_norm.yaml, crypt_four.yaml).  A list that names the same three
+// kernels in another order runs the same instantiation: perm[c] = position in the list of built kernel c.
+constexpr KernelId kBuiltTriples[3][3] = {{K_IM2COL, K_MAXPOOL, K_BNSTATS}, {K_MAXPOOL, K_HISTC, K_BNSTATS},
+                                          {K_BLAKE2B, K_SHA256D, K_ETHASH}};
+bool built_triple(const KernelId ids[3], int perm[3]) {
+  for (const auto &t : kBuiltTriples) {
+    bool all = true;
+    for (int c = 0; c < 3 && all; c++) {
+      perm[c] = -1;
+      for (int i = 0; i < 3; i++)
+        if (ids[i] == t[c]) perm[c] = i;
+      all = perm[c] >= 0;
+    }
+    if (all) return true;
+  }
+  return false;
 }
 
 // The reference's Context partitions a block among any number of kernels (include/KernelFusion.h:45-80);
@@ -743,6 +764,11 @@ HF_API int hf_plan_create(const hf_config *cfg, int fusion_index, const char *pr
     if (split_threads > 0) {
       return fail(HF_EINVAL, "split_threads shapes a pair; give a three-kernel plan its block with hf_plan_set_block_n");
     }
+    int perm[3];
+    if (!built_triple(plan->ids, perm)) {
+      return fail(HF_EUNSUPPORTED, "three-kernel fusions are built for im2col + max-pool + bn-stats, max-pool + histogram + "
+                                   "bn-stats and ccminer-Blake2b + SHA-256d + Ethash (in any order); this list is none of them");
+    }
     if (f.split || f.threads || f.lending >= 0 || f.barrier >= 0 || f.launch_bound >= 0) {
       return fail(HF_EINVAL, "fusion '" + f.file + "': Split / Threads / Lending / Barrier / LaunchBound shape a pair; a three-kernel entry takes 'Blocks'");
     }
@@ -810,15 +836,17 @@ HF_API int hf_plan_create(const hf_config *cfg, int fusion_index, const char *pr
   if (is_crypto(plan->ids[0]) && !p->base_line && plan->part.launch_threads > 512) {
     return fail(HF_EINVAL, "search kernels are built for fused blocks of at most 512 threads");
   }
-  if (f.lending >= 0) plan->lending = f.lending != 0;
-  if (f.launch_bound >= 0 && split_idx == HF_SPLIT_TABLE) plan->bounded = f.launch_bound;
+  // the entry's tuned keys belong to its tuned shape: a plan of an explicit split or variant starts from the library's defaults
+  const bool table_shape = split_idx == HF_SPLIT_TABLE && split_threads <= 0;
+  if (f.lending >= 0 && table_shape) plan->lending = f.lending != 0;
+  if (f.launch_bound >= 0 && table_shape) plan->bounded = f.launch_bound;
   const bool b1 = body_has_barriers(plan->ids[0]), b2 = body_has_barriers(plan->ids[1]);
   // One barrier policy per pair: nothing to do when neither body synchronises;
   // an LDS-counter barrier scoped to the synchronising half otherwise.  (Both
   // tensor bodies that synchronise do so twice per block, so a pair of them may
   // also share the hardware barrier: HF_BARRIER_MATCHED via hf_plan_set_barrier_mode.)
   plan->barrier_mode = (b1 || b2) ? HF_BARRIER_SUBSET : HF_BARRIER_NONE;
-  if (f.barrier >= 0 && !p->base_line) {
+  if (f.barrier >= 0 && !p->base_line && table_shape) {
     rc = hf_plan_set_barrier_mode(plan.get(), f.barrier);
     if (rc != HF_OK) {
       return rc;
@@ -1404,9 +1432,25 @@ int do_launch_fused3(const hf_plan *plan, const Prepared *p, int grid_blocks, hi
   const unsigned long long threads = (unsigned long long)grid * block;
   if (threads > 0xFFFFFFFFull || !counter_fits(p[0], threads) || !counter_fits(p[1], threads) || !counter_fits(p[2], threads))
     return fail(HF_EINVAL, kCounterMsg);
-  const void *const blobs[3] = {p[0].blob, p[1].blob, p[2].blob};
-  const hipError_t e = is_crypto(plan->ids[0]) ? launch_fused3_crypto(plan->ids, vertical, blobs, g, grid, block, lds, stream)
-                                               : launch_fused3_dl(plan->ids, vertical, blobs, g, grid, block, lds, stream);
+  // into the order the instantiation is built in: kernel c of it is the list's kernel perm[c]
+  int perm[3];
+  if (!built_triple(plan->ids, perm)) return fail(HF_EUNSUPPORTED, "this three-kernel list is not built");
+  FuseGeom3 b;
+  KernelId ids[3];
+  const void *blobs[3];
+  for (int c = 0; c < 3; c++) {
+    const int i = perm[c];
+    ids[c] = plan->ids[i];
+    blobs[c] = p[i].blob;
+    b.lo[c] = vertical ? 0u : plan->part.lo[i];
+    b.d[c] = g.d[i];
+    b.lds[c] = g.lds[i];
+    b.hint[c] = g.hint[i];
+    b.grid[c] = g.grid[i];
+  }
+  const bool bounded = plan_build_waves(plan) != 0;   // the launch-bound presets: the build bounded for 8 waves per SIMD
+  const hipError_t e = is_crypto(ids[0]) ? launch_fused3_crypto(ids, vertical, bounded, blobs, b, grid, block, lds, stream)
+                                         : launch_fused3_dl(ids, vertical, bounded, blobs, b, grid, block, lds, stream);
   if (e == hipErrorNotSupported) return fail(HF_EUNSUPPORTED, "this three-kernel list is not built (built: the reference's lists, in their order)");
   if (e != hipSuccess) return hip_fail(e, "fused launch");
   return HF_OK;
@@ -1471,6 +1515,57 @@ HF_API int hf_copy_f32(const float *src, float *dst, uint64_t n, void *stream) t
   hipError_t e = launch_copy_f32(src, dst, n, static_cast<hipStream_t>(stream));
   if (e != hipSuccess) return hip_fail(e, "copy launch");
   return HF_OK;
+} catch (...) {
+  return trap_exception();
+}
+
+namespace {
+int check_stream_probe(int pattern, const void *src, void *dst, uint64_t bytes, int grid_blocks, int block_threads) {
+  if (pattern < HF_STREAM_EMPTY || pattern > HF_STREAM_WRITE_XCD) return fail(HF_EINVAL, "unknown stream pattern");
+  if (pattern == HF_STREAM_EMPTY) return HF_OK;
+  const bool writes_only = pattern == HF_STREAM_WRITE || pattern == HF_STREAM_WRITE_STRIDED || pattern == HF_STREAM_WRITE_XCD;
+  const bool reads_only = pattern == HF_STREAM_READ || pattern == HF_STREAM_READ_LINES;
+  if ((!writes_only && !src) || !dst) return fail(HF_EINVAL, "null pointer");
+  if ((!writes_only && !aligned16(src)) || (!reads_only && !aligned16(dst))) return fail(HF_EINVAL, "buffers must be 16-byte aligned");
+  if (grid_blocks <= 0 || block_threads <= 0 || block_threads % (int)kWave || block_threads > (int)kMaxBlock)
+    return fail(HF_EINVAL, "grid must be positive and the block a multiple of 64 up to 1024");
+  if (pattern == HF_STREAM_WRITE_XCD && grid_blocks % 8) return fail(HF_EINVAL, "the XCD-ordered pattern needs a multiple of eight workgroups");
+  const uint64_t threads = (uint64_t)grid_blocks * (uint64_t)block_threads;
+  // whole vectors, shared out evenly: every workgroup (every thread, for the random lines) gets the same share
+  const uint64_t unit = 16ull * (pattern == HF_STREAM_READ_LINES ? threads * 4ull : (uint64_t)grid_blocks);
+  if (bytes == 0 || bytes % unit)
+    return fail(HF_EINVAL, "bytes must be a positive multiple of 16 * grid (64 * grid * block for the random lines)");
+  if (pattern == HF_STREAM_READ_LINES && (bytes >> 7) > 0xFFFFFFFFull) return fail(HF_EINVAL, "more than 2^32 lines");
+  return HF_OK;
+}
+}  // namespace
+
+HF_API int hf_stream_probe(int pattern, const void *src, void *dst, uint64_t bytes, int grid_blocks, int block_threads,
+                           void *stream) try {
+  if (int rc = check_stream_probe(pattern, src, dst, bytes, grid_blocks, block_threads)) return rc;
+  hipError_t e = launch_stream_probe(pattern, src, dst, bytes / 16, (unsigned)grid_blocks, (unsigned)block_threads,
+                                     static_cast<hipStream_t>(stream));
+  if (e != hipSuccess) return hip_fail(e, "stream probe launch");
+  return HF_OK;
+} catch (...) {
+  return trap_exception();
+}
+
+HF_API int hf_time_stream_probe(int pattern, const void *src, void *dst, uint64_t bytes, uint64_t src_stride,
+                                uint64_t dst_stride, int nbuf, int grid_blocks, int block_threads, int warmup, int iters,
+                                void *stream_, float *elapsed_ms) try {
+  if (!elapsed_ms) return fail(HF_EINVAL, "null argument");
+  if (nbuf <= 0 || iters <= 0 || warmup < 0 || src_stride % 16 || dst_stride % 16) return fail(HF_EINVAL, "bad repetition arguments");
+  if (int rc = check_stream_probe(pattern, src, dst, bytes, grid_blocks, block_threads)) return rc;
+  hipStream_t stream = static_cast<hipStream_t>(stream_);
+  auto once = [&](int r) -> int {
+    const uint64_t k = (uint64_t)(r % nbuf);
+    const void *s = src ? static_cast<const char *>(src) + k * src_stride : nullptr;
+    void *d = dst ? static_cast<char *>(dst) + k * dst_stride : nullptr;
+    hipError_t e = launch_stream_probe(pattern, s, d, bytes / 16, (unsigned)grid_blocks, (unsigned)block_threads, stream);
+    return e == hipSuccess ? HF_OK : hip_fail(e, "stream probe launch");
+  };
+  return time_repetitions(stream, warmup, iters, once, elapsed_ms);
 } catch (...) {
   return trap_exception();
 }

@@ -761,7 +761,7 @@ struct HistcBody {
   // The input stream: 16-byte non-temporal loads (values made up from the address in the loads-off timing build).
   static __device__ __forceinline__ f32x4 ldh(const float *p) {
     if (HF_TAKEAPART & 8) {
-      const float f = __builtin_amdgcn_fractf((float)((unsigned)(size_t)p >> 4) * 0.6180339887f);  // full-rate ops only
+      const float f = __builtin_amdgcn_fractf((float)(((unsigned)(size_t)p >> 4) & 0xFFFFu) * 0.6180339887f);  // full-rate ops only
       return f32x4{f, __builtin_amdgcn_fractf(f + 0.3819f), __builtin_amdgcn_fractf(f + 0.7071f), __builtin_amdgcn_fractf(f + 0.1234f)};
     }
     return ld4_stream(p);

@@ -49,25 +49,34 @@ enum KernelId {
   K_COUNT
 };
 
-// Register-bounded builds.  Every pair has one for kBoundedWaves waves per SIMD; the pairs of the
-// shipped list whose occupancy formula (min over the kernels of regfile / Reg / threads, capped by the
-// resident threads: lib/KernelFuser/KernelPrinter.cpp:44-66, with this part's 128 K registers and
-// 2048 threads per CU) asks for fewer waves at their shipped block shape have a second build at exactly
-// that bound.
+// Register-bounded builds.  The reference prints `__launch_bounds__(T, B)` with B = min over the kernels of
+// regfile / Reg / threads, capped by the resident threads (lib/KernelFuser/KernelPrinter.cpp:44-66): B blocks of T
+// threads are to fit a multiprocessor.  With this part's 128 K registers and 2048 threads per CU that is a bound of
+// ceil(B * T / 64 / 4) waves per SIMD.  Every pair has a build for kBoundedWaves waves per SIMD.  The five benchmarked
+// pairs have one for each of 5, 6, 7 and 8, so that whatever block shape a plan of theirs is given, the build a
+// launch-bound preset runs is bounded at exactly the formula's value (up to four waves per SIMD the plain build's
+// launch bound already holds); three more pairs of the shipped list have a second build at the value of their
+// shipped shape.
 constexpr int kBoundedWaves = 8;
+constexpr int kMinSetWaves = 5;
+constexpr bool pair_has_wave_set(KernelId k1, KernelId k2) {
+  return (k1 == K_IM2COL && k2 == K_MAXPOOL) || (k1 == K_BNSTATS && k2 == K_UPSAMPLE_NEAREST) ||
+         (k1 == K_HISTC && k2 == K_MAXPOOL) || (k1 == K_SHA256D && k2 == K_SIA_BLAKE2B) ||
+         (k1 == K_ETHASH && k2 == K_SIA_BLAKE2B);
+}
 constexpr int pair_extra_waves(KernelId k1, KernelId k2) {
-  return (k1 == K_IM2COL && k2 == K_MAXPOOL) ? 5                // 2 blocks of 256 + 448 threads
-         : (k1 == K_HISTC && k2 == K_MAXPOOL) ? 7               // 2 blocks of 768 + 128
-         : (k1 == K_ETHASH && k2 == K_SIA_BLAKE2B) ? 6          // 8 blocks of 128 + 64
-         : (k1 == K_IM2COL && k2 == K_HISTC) ? 7                // 2 blocks of 640 + 256
+  return (k1 == K_IM2COL && k2 == K_HISTC) ? 7                  // 2 blocks of 640 + 256 threads
          : (k1 == K_IM2COL && k2 == K_UPSAMPLE_NEAREST) ? 6     // 2 blocks of 256 + 512
-         : (k1 == K_MAXPOOL && k2 == K_BNSTATS) ? 7             // 9 blocks of 64 + 128
          : (k1 == K_IM2COL && k2 == K_UPSAMPLE_BILINEAR) ? 6    // 2 blocks of 256 + 512
                                                          : 0;
 }
-// The bound of the build that runs when `waves` waves per SIMD are asked for (0: the plain build).
+// The bound of the build that runs when `waves` waves per SIMD are asked for (0: the plain build): the smallest
+// built bound that is not below the request.
 constexpr int built_bound_waves(KernelId k1, KernelId k2, int waves) {
-  return waves <= 0 ? 0 : (pair_extra_waves(k1, k2) != 0 && waves <= pair_extra_waves(k1, k2)) ? pair_extra_waves(k1, k2) : kBoundedWaves;
+  return waves <= 0 ? 0
+         : pair_has_wave_set(k1, k2) ? (waves < kMinSetWaves ? kMinSetWaves : waves > kBoundedWaves ? kBoundedWaves : waves)
+         : (pair_extra_waves(k1, k2) != 0 && waves <= pair_extra_waves(k1, k2)) ? pair_extra_waves(k1, k2)
+                                                                                : kBoundedWaves;
 }
 
 
@@ -306,11 +315,14 @@ void vertical_kernel_lb(typename K1::Args a1, typename K2::Args a2, FuseGeom g) 
 // ----------------------------------------------------------------------------
 // Three kernels in one workgroup (the reference's Context partitions a block among any number of
 // kernels, include/KernelFusion.h:45-80; configs/crypt_four.yaml and im2col_maxpool_norm.yaml
-// list three).  Waves [0, d0/64) run kernel 0, the next d1/64 kernel 1, the rest kernel 2.  Each
+// list three).  Kernel k runs on threads [lo[k], lo[k] + d[k]): in the order a list is built in that is waves
+// [0, d0/64), the next d1/64 and the rest; a list that names the same kernels in another order is the same
+// instantiation with other bounds and the arguments in the built order.  Each
 // kernel strides over its own number of workgroups; in a block beyond that number its waves end at
 // once (no lending here).  A body that synchronises uses its own LDS arrival counter.
 // ----------------------------------------------------------------------------
 struct FuseGeom3 {
+  unsigned lo[3];    // first thread of each part (the parts follow the fusion list's order, the kernels the built order)
   unsigned d[3];     // threads of each part
   unsigned lds[3];   // LDS bytes of each part
   unsigned hint[3];  // fast-path selectors
@@ -325,9 +337,9 @@ __device__ __forceinline__ void run_part(const typename K::Args &a, unsigned tid
   K::run(a, sb, lds, hint);
 }
 
-template <class K0, class K1, class K2, int T>
-__global__ __launch_bounds__(T) void fused_kernel3(typename K0::Args a0, typename K1::Args a1, typename K2::Args a2,
-                                                   FuseGeom3 g) {
+template <class K0, class K1, class K2>
+__device__ __forceinline__ void fused_block3(const typename K0::Args &a0, const typename K1::Args &a1,
+                                             const typename K2::Args &a2, const FuseGeom3 &g) {
   extern __shared__ __align__(16) unsigned char smem[];
   unsigned *bars = reinterpret_cast<unsigned *>(smem);
   const unsigned tid = threadIdx.x, bid = blockIdx.x;
@@ -336,22 +348,34 @@ __global__ __launch_bounds__(T) void fused_kernel3(typename K0::Args a0, typenam
     if (tid < kBarrierWords) bars[tid] = 0;
     __syncthreads();
   }
-  const unsigned wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-  const unsigned w0 = g.d[0] >> 6, w1 = w0 + (g.d[1] >> 6);
+  const unsigned first = __builtin_amdgcn_readfirstlane(tid & ~63u);   // this wave's first thread: the selector is a scalar
   unsigned char *l0 = smem + 4 * kBarrierWords, *l1 = l0 + g.lds[0], *l2 = l1 + g.lds[1];
-  if (wave < w0)
-    run_part<K0, K0::kBarriers ? BAR_SUBSET : BAR_WORKGROUP>(a0, tid, g.d[0], bid, g.grid[0], bars + 0, l0, g.hint[0]);
-  else if (wave < w1)
-    run_part<K1, K1::kBarriers ? BAR_SUBSET : BAR_WORKGROUP>(a1, tid - g.d[0], g.d[1], bid, g.grid[1], bars + 1, l1, g.hint[1]);
-  else
-    run_part<K2, K2::kBarriers ? BAR_SUBSET : BAR_WORKGROUP>(a2, tid - g.d[0] - g.d[1], g.d[2], bid, g.grid[2], bars + 2, l2,
+  if (first - g.lo[0] < g.d[0])
+    run_part<K0, K0::kBarriers ? BAR_SUBSET : BAR_WORKGROUP>(a0, tid - g.lo[0], g.d[0], bid, g.grid[0], bars + 0, l0, g.hint[0]);
+  else if (first - g.lo[1] < g.d[1])
+    run_part<K1, K1::kBarriers ? BAR_SUBSET : BAR_WORKGROUP>(a1, tid - g.lo[1], g.d[1], bid, g.grid[1], bars + 1, l1, g.hint[1]);
+  else if (first - g.lo[2] < g.d[2])
+    run_part<K2, K2::kBarriers ? BAR_SUBSET : BAR_WORKGROUP>(a2, tid - g.lo[2], g.d[2], bid, g.grid[2], bars + 2, l2,
                                                              g.hint[2]);
 }
 
-// The vertical baseline of a three-kernel list: a block of max(d) threads runs the bodies one after the other.
 template <class K0, class K1, class K2, int T>
-__global__ __launch_bounds__(T) void vertical_kernel3(typename K0::Args a0, typename K1::Args a1, typename K2::Args a2,
-                                                      FuseGeom3 g) {
+__global__ __launch_bounds__(T) void fused_kernel3(typename K0::Args a0, typename K1::Args a1, typename K2::Args a2,
+                                                   FuseGeom3 g) {
+  fused_block3<K0, K1, K2>(a0, a1, a2, g);
+}
+
+// The launch-bound presets of a three-kernel list: the same kernel compiled for kBoundedWaves waves per SIMD.
+template <class K0, class K1, class K2, int T>
+__global__ __launch_bounds__(T) __attribute__((amdgpu_waves_per_eu(kBoundedWaves, kBoundedWaves)))
+void fused_kernel3_lb(typename K0::Args a0, typename K1::Args a1, typename K2::Args a2, FuseGeom3 g) {
+  fused_block3<K0, K1, K2>(a0, a1, a2, g);
+}
+
+// The vertical baseline of a three-kernel list: a block of max(d) threads runs the bodies one after the other.
+template <class K0, class K1, class K2>
+__device__ __forceinline__ void vertical_block3(const typename K0::Args &a0, const typename K1::Args &a1,
+                                                const typename K2::Args &a2, const FuseGeom3 &g) {
   extern __shared__ __align__(16) unsigned char smem[];
   unsigned *bars = reinterpret_cast<unsigned *>(smem);
   const unsigned tid = threadIdx.x, bid = blockIdx.x;
@@ -368,6 +392,18 @@ __global__ __launch_bounds__(T) void vertical_kernel3(typename K0::Args a0, type
     run_part<K1, K1::kBarriers ? BAR_SUBSET : BAR_WORKGROUP>(a1, tid, g.d[1], bid, g.grid[1], bars + 1, l1, g.hint[1]);
   if (wave < (g.d[2] >> 6))
     run_part<K2, K2::kBarriers ? BAR_SUBSET : BAR_WORKGROUP>(a2, tid, g.d[2], bid, g.grid[2], bars + 2, l2, g.hint[2]);
+}
+
+template <class K0, class K1, class K2, int T>
+__global__ __launch_bounds__(T) void vertical_kernel3(typename K0::Args a0, typename K1::Args a1, typename K2::Args a2,
+                                                      FuseGeom3 g) {
+  vertical_block3<K0, K1, K2>(a0, a1, a2, g);
+}
+
+template <class K0, class K1, class K2, int T>
+__global__ __launch_bounds__(T) __attribute__((amdgpu_waves_per_eu(kBoundedWaves, kBoundedWaves)))
+void vertical_kernel3_lb(typename K0::Args a0, typename K1::Args a1, typename K2::Args a2, FuseGeom3 g) {
+  vertical_block3<K0, K1, K2>(a0, a1, a2, g);
 }
 
 }  // namespace hfuse

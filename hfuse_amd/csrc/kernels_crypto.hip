@@ -29,19 +29,27 @@ hipError_t pair(FuseMode mode, int waves, const void *a1, const void *a2, const 
   const bool bounded = build != 0;
   switch (mode) {
     case MODE_HFUSE:
+      if constexpr (pair_has_wave_set(K1::kId, K2::kId)) {
+        // one build per bound a block shape of this pair can ask for
+        switch (build) {
+          case 0: hipLaunchKernelGGL((fused_kernel<K1, K2, kCryptoBlock, false>), dim3(grid), dim3(g.d1 + g.d2), lds, s, x1, x2, g); break;
+          case 5: hipLaunchKernelGGL((fused_kernel_lb<K1, K2, kCryptoBlock, false, 5>), dim3(grid), dim3(g.d1 + g.d2), lds, s, x1, x2, g); break;
+          case 6: hipLaunchKernelGGL((fused_kernel_lb<K1, K2, kCryptoBlock, false, 6>), dim3(grid), dim3(g.d1 + g.d2), lds, s, x1, x2, g); break;
+          case 7: hipLaunchKernelGGL((fused_kernel_lb<K1, K2, kCryptoBlock, false, 7>), dim3(grid), dim3(g.d1 + g.d2), lds, s, x1, x2, g); break;
+          default: hipLaunchKernelGGL((fused_kernel_lb<K1, K2, kCryptoBlock, false, 8>), dim3(grid), dim3(g.d1 + g.d2), lds, s, x1, x2, g); break;
+        }
+        break;
+      }
       if constexpr (kExtra != 0) {
         if (build == kExtra) {
-          hipLaunchKernelGGL((fused_kernel_lb<K1, K2, kCryptoBlock, false, kExtra>), dim3(grid), dim3(g.d1 + g.d2), lds, s,
-                             x1, x2, g);
+          hipLaunchKernelGGL((fused_kernel_lb<K1, K2, kCryptoBlock, false, kExtra>), dim3(grid), dim3(g.d1 + g.d2), lds, s, x1, x2, g);
           break;
         }
       }
-      if (bounded)
-        hipLaunchKernelGGL((fused_kernel_lb<K1, K2, kCryptoBlock, false>), dim3(grid), dim3(g.d1 + g.d2), lds, s, x1,
-                           x2, g);
+      if (build)
+        hipLaunchKernelGGL((fused_kernel_lb<K1, K2, kCryptoBlock, false>), dim3(grid), dim3(g.d1 + g.d2), lds, s, x1, x2, g);
       else
-        hipLaunchKernelGGL((fused_kernel<K1, K2, kCryptoBlock, false>), dim3(grid), dim3(g.d1 + g.d2), lds, s, x1, x2,
-                           g);
+        hipLaunchKernelGGL((fused_kernel<K1, K2, kCryptoBlock, false>), dim3(grid), dim3(g.d1 + g.d2), lds, s, x1, x2, g);
       break;
     case MODE_MATCHED:
       return hipErrorNotSupported;  // none of the searches has a barrier
@@ -75,16 +83,22 @@ hipError_t launch_native_crypto(KernelId k, const void *args, unsigned hint, uns
 }
 
 // The three-kernel list of configs/crypt_four.yaml, in its listed order.
-hipError_t launch_fused3_crypto(const KernelId k[3], bool vertical, const void *const a[3], const FuseGeom3 &g, unsigned grid,
-                                unsigned block, size_t lds, hipStream_t s) {
+hipError_t launch_fused3_crypto(const KernelId k[3], bool vertical, bool bounded, const void *const a[3], const FuseGeom3 &g,
+                                unsigned grid, unsigned block, size_t lds, hipStream_t s) {
   if (!(k[0] == K_BLAKE2B && k[1] == K_SHA256D && k[2] == K_ETHASH)) return hipErrorNotSupported;
   if (block > (unsigned)kCryptoBlock) return hipErrorNotSupported;
   const auto &x0 = *static_cast<const Blake2bDevArgs *>(a[0]);
   const auto &x1 = *static_cast<const Sha256dDevArgs *>(a[1]);
   const auto &x2 = *static_cast<const EthashDevArgs *>(a[2]);
-  if (vertical)
+  if (vertical && bounded)
+    hipLaunchKernelGGL((vertical_kernel3_lb<CcminerBlake2bBody, Sha256dBody, EthashBody, kCryptoBlock>), dim3(grid), dim3(block),
+                       lds, s, x0, x1, x2, g);
+  else if (vertical)
     hipLaunchKernelGGL((vertical_kernel3<CcminerBlake2bBody, Sha256dBody, EthashBody, kCryptoBlock>), dim3(grid), dim3(block),
                        lds, s, x0, x1, x2, g);
+  else if (bounded)
+    hipLaunchKernelGGL((fused_kernel3_lb<CcminerBlake2bBody, Sha256dBody, EthashBody, kCryptoBlock>), dim3(grid), dim3(block), lds,
+                       s, x0, x1, x2, g);
   else
     hipLaunchKernelGGL((fused_kernel3<CcminerBlake2bBody, Sha256dBody, EthashBody, kCryptoBlock>), dim3(grid), dim3(block), lds,
                        s, x0, x1, x2, g);

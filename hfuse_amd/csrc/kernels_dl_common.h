@@ -32,6 +32,17 @@ hipError_t dl_pair(FuseMode mode, int waves, const void *a1, const void *a2, con
   const int build = built_bound_waves(K1::kId, K2::kId, waves);
   switch (mode) {
     case MODE_HFUSE:
+      if constexpr (pair_has_wave_set(K1::kId, K2::kId)) {
+        // one build per bound a block shape of this pair can ask for
+        switch (build) {
+          case 0: hipLaunchKernelGGL((fused_kernel<K1, K2, kDlBlock, false>), dim3(grid), dim3(g.d1 + g.d2), lds, s, x1, x2, g); break;
+          case 5: hipLaunchKernelGGL((fused_kernel_lb<K1, K2, kDlBlock, false, 5>), dim3(grid), dim3(g.d1 + g.d2), lds, s, x1, x2, g); break;
+          case 6: hipLaunchKernelGGL((fused_kernel_lb<K1, K2, kDlBlock, false, 6>), dim3(grid), dim3(g.d1 + g.d2), lds, s, x1, x2, g); break;
+          case 7: hipLaunchKernelGGL((fused_kernel_lb<K1, K2, kDlBlock, false, 7>), dim3(grid), dim3(g.d1 + g.d2), lds, s, x1, x2, g); break;
+          default: hipLaunchKernelGGL((fused_kernel_lb<K1, K2, kDlBlock, false, 8>), dim3(grid), dim3(g.d1 + g.d2), lds, s, x1, x2, g); break;
+        }
+        break;
+      }
       if constexpr (kExtra != 0) {
         if (build == kExtra) {
           hipLaunchKernelGGL((fused_kernel_lb<K1, K2, kDlBlock, false, kExtra>), dim3(grid), dim3(g.d1 + g.d2), lds, s, x1, x2, g);

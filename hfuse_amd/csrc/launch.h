@@ -28,13 +28,17 @@ hipError_t launch_fused_crypto(KernelId k1, KernelId k2, FuseMode mode, int wave
                                const FuseGeom &g, unsigned grid, size_t lds, hipStream_t stream);
 
 // Three-kernel fusions (vertical = the baseline preset).  hipErrorNotSupported when the list is not instantiated.
-hipError_t launch_fused3_dl(const KernelId k[3], bool vertical, const void *const a[3], const FuseGeom3 &g, unsigned grid,
-                            unsigned block, size_t lds, hipStream_t stream);
-hipError_t launch_fused3_crypto(const KernelId k[3], bool vertical, const void *const a[3], const FuseGeom3 &g, unsigned grid,
-                                unsigned block, size_t lds, hipStream_t stream);
+// `bounded`: the build compiled for 8 waves per SIMD (the launch-bound presets).
+hipError_t launch_fused3_dl(const KernelId k[3], bool vertical, bool bounded, const void *const a[3], const FuseGeom3 &g,
+                            unsigned grid, unsigned block, size_t lds, hipStream_t stream);
+hipError_t launch_fused3_crypto(const KernelId k[3], bool vertical, bool bounded, const void *const a[3], const FuseGeom3 &g,
+                                unsigned grid, unsigned block, size_t lds, hipStream_t stream);
 
 hipError_t launch_fill_splitmix64(unsigned long long *dst, unsigned long long nwords, unsigned long long seed,
                                   hipStream_t stream);
 hipError_t launch_copy_f32(const float *src, float *dst, unsigned long long n, hipStream_t stream);
+// The bare stream kernels (HF_STREAM_* patterns) over n4 16-byte vectors.
+hipError_t launch_stream_probe(int pattern, const void *src, void *dst, unsigned long long n4, unsigned grid, unsigned block,
+                               hipStream_t stream);
 
 }  // namespace hfuse

@@ -127,8 +127,32 @@ struct Parser {
           if (!parse_seq(indent, child)) return false;  // sequence at the key's own column
         }
       } else {
-        child.kind = YamlNode::Scalar;
-        child.scalar = unquote(val);
+        const std::string v = unquote(val);
+        if (v.size() >= 2 && v.front() == '[' && v.back() == ']' && val.find('"') == std::string::npos &&
+            val.find('\'') == std::string::npos) {
+          // a flow sequence of plain scalars on the key's line: `Blocks: [768, 768]`
+          child.kind = YamlNode::Seq;
+          const std::string inner = v.substr(1, v.size() - 2);
+          if (inner.find('[') != std::string::npos || inner.find('{') != std::string::npos)
+            return fail(ln.no, "nested flow collections are not read");
+          for (size_t a = 0; a <= inner.size();) {
+            size_t e = inner.find(',', a);
+            if (e == std::string::npos) e = inner.size();
+            YamlNode item;
+            item.kind = YamlNode::Scalar;
+            item.line = ln.no;
+            item.scalar = unquote(inner.substr(a, e - a));
+            if (item.scalar.empty()) {
+              if (e == inner.size() && child.seq.empty() && unquote(inner).empty()) break;  // `[]`
+              return fail(ln.no, "empty item in a flow sequence");
+            }
+            child.seq.push_back(std::move(item));
+            a = e + 1;
+          }
+        } else {
+          child.kind = YamlNode::Scalar;
+          child.scalar = v;
+        }
         if (pos < lines.size() && lines[pos].indent > indent)
           return fail(lines[pos].no, "unexpected indentation after scalar value");
       }

@@ -4,9 +4,13 @@ The reference generates one fused kernel per split of the enumeration 128*(n+1) 
 (tools/llvm-smart-fuser/main.cpp:215-236), builds and profiles each, and keeps the fastest.
 Here every split is a launch-time choice of the same compiled kernel, so the sweep is a loop of
 timed launches: block shapes (threads of kernel 1, threads of kernel 2) in wavefront multiples,
-wave lending on and off, and the barrier modes legal for the pair.  The winner is written back
-into the fusion list as the `Split:` / `Threads:` / `Lending:` / `Barrier:` / `LaunchBound:` keys
-the library applies when a plan is created with the table split.
+wave lending on and off, and the barrier modes legal for the pair.  The reference prints its vertical
+presets next to the horizontal ones and the user keeps whichever profiles fastest (main.cpp:182-193), so
+the sweep also times the vertical kernel: the threads that run each body and the workgroups each body
+strides over (a few resident blocks whose threads take the two kernels' work in turn).  The winner is
+written back into the fusion list as the `Split:` / `Threads:` / `Lending:` / `Barrier:` / `LaunchBound:`
+keys the library applies when a plan is created with the table split, and, where a vertical form wins,
+`Preset: vfuse` with its `Blocks:` and `Grids:` (the entry keeps the keys of its best thread partition too).
 
 The register-cap half of the reference's experiments (its *_lb presets, `Reg` bound per
 kernel): a gfx950 kernel's VGPR budget is fixed at compile time, so the library carries two
@@ -43,9 +47,14 @@ class Candidate:
     barrier_mode: Optional[int] = None   # None: the library's choice for the pair
     grids: Tuple[int, int] = (0, 0)      # (0, 0): the library's grids
     bounded: bool = False                # the register-bounded build (the reference's *_lb presets)
+    preset: str = "hfuse"                # "vfuse": both bodies from thread 0, threads1 / threads2 run each
+
+    @property
+    def vertical(self) -> bool:
+        return self.preset.startswith("vfuse")
 
     def label(self) -> str:
-        s = f"{self.threads1}+{self.threads2}"
+        s = f"{self.threads1}+{self.threads2}" if not self.vertical else f"vfuse {self.threads1}|{self.threads2}"
         if not self.lending:
             s += " nolend"
         if self.barrier_mode is not None:
@@ -66,6 +75,8 @@ class TuneResult:
     t_table_ms: float                 # the untuned table split of the kernel table
     t_b2b_ms: float                   # the two native launches back to back
     table: List[Tuple[str, float]] = field(default_factory=list)   # (candidate label, ms) of the whole sweep
+    best_partition: Optional[Candidate] = None   # the fastest thread partition (== best unless a vertical form won)
+    t_partition_ms: float = float("nan")
 
     @property
     def speedup_pct(self) -> float:
@@ -100,15 +111,34 @@ SEARCH_NAMES = {"ethash_search", "ethash_search2", "ethash_search3", "ethash_sea
 
 
 def _make_plan(cfg: H.Config, fusion_index: int, c: Candidate) -> H.Plan:
-    plan = cfg.plan(fusion_index, "hfuse", L.HF_SPLIT_TABLE)
+    plan = cfg.plan(fusion_index, c.preset, L.HF_SPLIT_TABLE)
     plan.set_block(c.threads1, c.threads2)
-    plan.set_lending(c.lending)
-    if c.barrier_mode is not None:
-        plan.set_barrier_mode(c.barrier_mode)
-    if c.grids != (0, 0):
-        plan.set_grids(*c.grids)
+    if not c.vertical:
+        plan.set_lending(c.lending)
+        if c.barrier_mode is not None:
+            plan.set_barrier_mode(c.barrier_mode)
+    plan.set_grids(*c.grids)
     plan.set_launch_bound(c.bounded)
     return plan
+
+
+def vertical_candidates(cfg: H.Config, fusion_index: int, cus: int, max_block: int = MAX_TENSOR_BLOCK) -> List[Candidate]:
+    """Vertical forms of a pair: the same threads run both bodies, in blocks of 512 to 1024 threads, with the
+    library's own grids (every thread one or two items) and with one or two resident blocks per CU whose
+    threads stride over each kernel's work."""
+    _, k1, k2 = cfg.fusion(fusion_index)
+    y1, y2 = cfg.kernel(k1).block_dim.y, cfg.kernel(k2).block_dim.y
+    out = []
+    for t in (512, 768, 1024):
+        if t > max_block or t % y1 or t % y2:
+            continue
+        for per_cu in (0, 1, 2):
+            if per_cu * t > 2048:
+                continue
+            out.append(Candidate(t, t, grids=(per_cu * cus, per_cu * cus), preset="vfuse"))
+        out.append(Candidate(t, t, grids=(cus, 0), preset="vfuse"))   # kernel 1 on resident blocks, kernel 2 one item a thread
+        out.append(Candidate(t, t, grids=(0, cus), preset="vfuse"))
+    return out
 
 
 def tune(cfg: H.Config, fusion_index: int, args1: Sequence, args2: Sequence, *,
@@ -116,7 +146,7 @@ def tune(cfg: H.Config, fusion_index: int, args1: Sequence, args2: Sequence, *,
          barrier_modes: Sequence[Optional[int]] = (None,), grids: Sequence[Tuple[int, int]] = ((0, 0),),
          probe_iters: int = 20, final_iters: int = 100, finalists: int = 4, warmup: int = 3,
          grid_blocks=0, launch_bound: bool = True, verbose: bool = False,
-         rotation: Optional[H.Rotation] = None) -> TuneResult:
+         rotation: Optional[H.Rotation] = None, extra: Sequence[Candidate] = ()) -> TuneResult:
     """Sweep the candidates of one pair on the caller's argument sets and return the fastest.
 
     args1[i] / args2[i] are argument structs of independent buffer sets the timed launches rotate
@@ -136,7 +166,7 @@ def tune(cfg: H.Config, fusion_index: int, args1: Sequence, args2: Sequence, *,
     if blocks is None:
         blocks = block_candidates(cfg, fusion_index, step=2 * WAVE)
     cands = [Candidate(t1, t2, ln, bm, g) for (t1, t2) in blocks for ln in lending for bm in barrier_modes
-             for g in grids]
+             for g in grids] + list(extra)
     probed = []
     for c in cands:
         try:
@@ -151,6 +181,8 @@ def tune(cfg: H.Config, fusion_index: int, args1: Sequence, args2: Sequence, *,
         raise RuntimeError(f"no legal candidate for {k1} + {k2}")
     probed.sort(key=lambda r: r[0])
     final = probed[:max(1, finalists)]
+    if all(c.vertical for _, c, _ in final):      # keep the fastest thread partitions in the final as well
+        final += [r for r in probed if not r[1].vertical][:2]
     if launch_bound:
         import dataclasses
         for t, c, _ in list(final):
@@ -181,11 +213,14 @@ def tune(cfg: H.Config, fusion_index: int, args1: Sequence, args2: Sequence, *,
     near = [(t, i) for t, i in med if t <= med[0][0] * 1.005]
     t_best, ibest = min(near, key=lambda r: ((not final[r[1]][1].lending) + (final[r[1]][1].barrier_mode is not None)
                                              + final[r[1]][1].bounded, r[0]))
+    parts = [(t, i) for t, i in med if not final[i][1].vertical]
     return TuneResult(file=file, kernels=(k1, k2), best=final[ibest][1], t_best_ms=t_best,
                       t_table_ms=statistics.median(s_table) if s_table else float("nan"),
                       t_b2b_ms=statistics.median(s_b2b),
                       table=[(c.label(), t) for t, c, _ in probed] +
-                            [(final[i][1].label(), t) for t, i in med if final[i][1].bounded])
+                            [(final[i][1].label(), t) for t, i in med if final[i][1].bounded],
+                      best_partition=final[parts[0][1]][1] if parts else None,
+                      t_partition_ms=parts[0][0] if parts else float("nan"))
 
 
 # ------------------------------------------------------------------ three-kernel entries
@@ -295,7 +330,7 @@ def tune_shipped_triples(out_path: str, verbose: bool = False, search_log2=(26, 
 
 
 # ------------------------------------------------------------------ fusion list rewriting
-_TUNED_KEY = re.compile(r"^\s+(Split|Threads|Lending|Barrier|LaunchBound)\s*:")
+_TUNED_KEY = re.compile(r"^\s+(Split|Threads|Lending|Barrier|LaunchBound|Preset|Grids|Blocks)\s*:")
 BARRIER_NAMES = {L.HF_BARRIER_NONE: "none", L.HF_BARRIER_MATCHED: "matched", L.HF_BARRIER_SUBSET: "subset",
                  L.HF_BARRIER_BLOCKIDX: "blockidx"}
 
@@ -319,15 +354,22 @@ def apply_to_fusion_yaml(text: str, tuned: dict) -> str:
             while entry and (not entry[-1].strip() or entry[-1].lstrip().startswith("#")):
                 tail.insert(0, entry.pop())
             c = tuned[n]
-            if c is not None:
-                entry.append(f"  Split: {c.threads1}")
-                entry.append(f"  Threads: {c.threads1 + c.threads2}")
-                if not c.lending:
+            part = c[1] if isinstance(c, tuple) else c      # (winner, best thread partition) or one candidate
+            c = c[0] if isinstance(c, tuple) else c
+            if part is not None and not part.vertical:
+                entry.append(f"  Split: {part.threads1}")
+                entry.append(f"  Threads: {part.threads1 + part.threads2}")
+                if not part.lending:
                     entry.append("  Lending: false")
-                if c.barrier_mode is not None:
-                    entry.append(f"  Barrier: {BARRIER_NAMES[c.barrier_mode]}")
-                if c.bounded:
+                if part.barrier_mode is not None:
+                    entry.append(f"  Barrier: {BARRIER_NAMES[part.barrier_mode]}")
+                if part.bounded:
                     entry.append("  LaunchBound: true")
+            if c is not None and c.vertical:
+                entry.append(f"  Preset: {c.preset}{'_lb' if c.bounded else ''}")
+                entry.append(f"  Blocks: [{c.threads1}, {c.threads2}]")
+            if c is not None and c.grids != (0, 0):
+                entry.append(f"  Grids: [{c.grids[0]}, {c.grids[1]}]")
             entry.extend(tail)
         out.extend(entry)
     if not starts:
@@ -359,6 +401,9 @@ def main(argv=None) -> int:
     ap.add_argument("--blockidx", action="store_true",
                     help="also try the block-index partition (each workgroup runs one of the two kernels), "
                          "written as 'Barrier: blockidx' where it wins")
+    ap.add_argument("--vertical", action="store_true",
+                    help="also try the vertical kernel (the reference's vfuse preset) in blocks of 512-1024 threads, with the "
+                         "library's grids and with one or two resident blocks per CU; written as 'Preset: vfuse' where it wins")
     ap.add_argument("--verbose", action="store_true")
     ap.add_argument("--triples", action="store_true",
                     help="tune the block shapes (`Blocks:`) of the shipped three-kernel list instead of the pairs")
@@ -395,8 +440,10 @@ def main(argv=None) -> int:
         if tensor:
             bench_variant = {v[:2]: v[2:] for v in W.BENCH_TENSOR_PAIRS.values()}.get((k1, k2), ("", ""))
             pair = W.build_pair(file, k1, k2, *bench_variant)
+            cus = torch.cuda.get_device_properties(0).multi_processor_count
             r = tune(cfg, i, pair.args1, pair.args2, blocks=blocks,
-                     barrier_modes=(None, L.HF_BARRIER_BLOCKIDX) if args.blockidx else (None,), verbose=args.verbose)
+                     barrier_modes=(None, L.HF_BARRIER_BLOCKIDX) if args.blockidx else (None,), verbose=args.verbose,
+                     extra=vertical_candidates(cfg, i, cus) if args.vertical else (), rotation=pair.rotation)
             del pair
         else:
             sp = W.SearchPair(k1, k2, args.search_log2,
@@ -405,8 +452,10 @@ def main(argv=None) -> int:
             # ethash scans grid * its-threads nonces: every block shape gets the grid for the same range
             eth = 0 if k1 == "ethash_search" else 1 if k2 == "ethash_search" else None
             grid = (lambda t1, t2: sp.nonces[eth] // (t1, t2)[eth]) if eth is not None else 0
+            vertical = [Candidate(t, t, preset="vfuse") for t in (64, 128, 256)] if args.vertical else []
             r = tune(cfg, i, [a1], [a2], blocks=blocks, lending=(True,), probe_iters=1, final_iters=2,
-                     warmup=0, grid_blocks=grid, verbose=args.verbose)
+                     warmup=0, grid_blocks=grid, verbose=args.verbose, extra=vertical,
+                     barrier_modes=(None, L.HF_BARRIER_BLOCKIDX) if args.blockidx else (None,))
             del sp
         torch.cuda.empty_cache()
         gain = (r.t_table_ms / r.t_best_ms - 1.0) * 100.0 if r.t_table_ms == r.t_table_ms else float("inf")
@@ -417,7 +466,7 @@ def main(argv=None) -> int:
         # the same pair may be listed more than once (the reference's lists repeat pairs): tune once, write all
         for j, (_, a, b) in enumerate(cfg.fusions()):
             if (a, b) == (k1, k2):
-                tuned[j] = r.best if keep else None
+                tuned[j] = (r.best, r.best_partition) if keep else None
     with open(args.out, "w") as f:
         f.write(apply_to_fusion_yaml(text, tuned))
     print(f"wrote {args.out} ({len(tuned)} entries tuned)", file=sys.stderr)

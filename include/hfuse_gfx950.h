@@ -499,6 +499,35 @@ HF_API int hf_fill_splitmix64(uint64_t *dst, uint64_t nwords, uint64_t seed, voi
 /* Plain device copy, the unit the HBM counters are calibrated against. */
 HF_API int hf_copy_f32(const float *src, float *dst, uint64_t n, void *stream);
 
+/*
+ * Bare stream kernels (no counterpart in the reference): what the memory system of this part delivers for the
+ * access patterns of the kernels above, measured by the benchmark in the same run as the kernels that are judged
+ * against them.  16-byte non-temporal accesses; `bytes` is what one launch reads (HF_STREAM_WRITE: writes).
+ *   HF_STREAM_EMPTY       an empty kernel (the cost of a launch); the other arguments are ignored
+ *   HF_STREAM_READ        every workgroup reads one contiguous share of `src`; `dst` = 4 bytes, never written
+ *   HF_STREAM_WRITE       every workgroup writes one contiguous share of `dst` (`bytes`); `src` is ignored
+ *   HF_STREAM_WRITE_STRIDED  the same bytes written by a grid-stride loop (the whole grid inside one window at a time)
+ *   HF_STREAM_WRITE_XCD   HF_STREAM_WRITE with the workgroups renumbered so that each of the eight XCDs owns one
+ *                         contiguous eighth of `dst` (the grid must be a multiple of eight)
+ *   HF_STREAM_READ_LINES  uniformly random 128-byte lines out of `src` (`bytes` large), eight lanes a line, `bytes`
+ *                         read in total: the DAG reads of ethash_search; `dst` = 4 bytes, never written
+ *   HF_STREAM_COPY_1_4    reads `bytes` from `src`, writes them to four planes of `dst` (4 * `bytes`): the shape of
+ *                         upsample_nearest2d_out_frame
+ * `bytes` must divide into whole 16-byte vectors per workgroup (per thread and trip for the random lines).
+ */
+enum { HF_STREAM_EMPTY = 0, HF_STREAM_READ = 1, HF_STREAM_WRITE = 2, HF_STREAM_READ_LINES = 3, HF_STREAM_COPY_1_4 = 4,
+       HF_STREAM_WRITE_STRIDED = 5, HF_STREAM_WRITE_XCD = 6 };
+HF_API int hf_stream_probe(int pattern, const void *src, void *dst, uint64_t bytes, int grid_blocks, int block_threads,
+                           void *stream);
+/*
+ * `warmup` untimed and `iters` timed launches of one pattern between two events on `stream`; launch r works on
+ * src + (r % nbuf) * src_stride and dst + (r % nbuf) * dst_stride (bytes), so that a rotation through more than the
+ * 256 MB memory-side cache holds reads from HBM.  *elapsed_ms = milliseconds of the `iters` launches.
+ */
+HF_API int hf_time_stream_probe(int pattern, const void *src, void *dst, uint64_t bytes, uint64_t src_stride,
+                                uint64_t dst_stride, int nbuf, int grid_blocks, int block_threads, int warmup, int iters,
+                                void *stream, float *elapsed_ms);
+
 #ifdef __cplusplus
 }
 #endif

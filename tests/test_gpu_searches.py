@@ -1,9 +1,12 @@
 """GPU parity of the nonce searches, native and fused, through the C-ABI: every
 found nonce, digest and (for Ethash) mix digest must equal the CPU oracle's."""
+import os
+
 import numpy as np
 import pytest
 import torch
 
+from hfuse_amd import _lib as L
 from hfuse_amd import launcher as H
 from oracle import oracle as O
 
@@ -243,8 +246,8 @@ def test_every_shipped_search_pair(cuda, cfg):
 
 
 def test_ethash_sia_bounded_builds(cuda, cfg):
-    """Ethash + Sia-Blake2b in its two register-bounded builds (6 waves per SIMD, the occupancy formula's value
-    for 128 + 64 threads, and 8) against the oracle."""
+    """Ethash + Sia-Blake2b in its register-bounded builds (6 waves per SIMD is the occupancy formula's value for
+    128 + 64 threads; 5, 7 and 8 are built as well) against the oracle."""
     n_items = 1 << 14
     dag = _dag(cuda, n_items, SEED)
     header, h2 = O.seeded_bytes(32, SEED + 30), O.seeded_bytes(80, SEED + 31)
@@ -258,9 +261,9 @@ def test_ethash_sia_bounded_builds(cuda, cfg):
     want1 = oracle_hits(O.ethash_search(None, SEED, n_items, header, 7, grid * share, target))
     want2 = oracle_hits(O.sia_search(h2, 0, 1 << 15, EASY10))
     assert want1[0] > 0 and want2[0] > 0
-    for waves in (0, 8):
+    for waves in (0, 5, 7, 8):
         plan.set_launch_waves(waves)
-        assert plan.launch_waves[1] == (6 if waves == 0 else 8)
+        assert plan.launch_waves[1] == (6 if waves == 0 else waves)
         r1, r2 = H.new_search_results(), H.new_search_results()
         plan.launch(H.ethash_args(r1, 7), H.blake2b_args(r2, 1 << 15, 0, EASY10), grid_blocks=grid)
         sync()
@@ -289,22 +292,35 @@ def test_three_search_kernels_in_one_launch(cuda):
     want_b = (len(want_b), sorted(want_b))
     want_s = oracle_hits(O.sha256d_search(hs, 17, count, EASY10))
     assert want_b[0] > 0 and want_s[0] > 0
-    for preset, block, grid in (("hfuse", None, 96), ("hfuse", (64, 128, 192), 64), ("hfuse_lb", None, 32), ("vfuse", None, 96)):
-        plan = t.plan(i, preset)
+    # the list as the reference orders it, and the same three kernels listed in two other orders (the Context partitions
+    # in list order, include/KernelFusion.h:45-80: same instantiation, other thread bounds, arguments in list order)
+    kernels_yaml = open(os.path.join(hfuse_amd.CONFIG_DIR, "gfx950_kernels.yaml")).read()
+    names = ("blake2b_gpu_hash", "sha256d_gpu_hash_shared", "ethash_search")
+    cases = [(t, i, (0, 1, 2), preset, block, grid)
+             for preset, block, grid in (("hfuse", None, 96), ("hfuse", (64, 128, 192), 64), ("hfuse_lb", None, 32), ("vfuse", None, 96))]
+    for order in ((2, 0, 1), (1, 2, 0)):
+        text = "- File: permuted\n  Kernels:\n" + "".join(f"    - {names[k]}\n" for k in order) + "  Blocks: [128, 64, 192]\n"
+        cases += [(H.Config(text, kernels_yaml), 0, order, "hfuse", None, 48), (H.Config(text, kernels_yaml), 0, order, "vfuse", None, 48)]
+    for conf, idx, order, preset, block, grid in cases:
+        plan = conf.plan(idx, preset)
         if block:
             plan.set_block_n(*block)
         plan.bind_constants(consts)
         q = plan.partition_n
-        share = q.hi[2] - q.lo[2]
+        pos = order.index(2)                        # where the list names Ethash
+        share = q.hi[pos] - q.lo[pos]
         want_e = oracle_hits(O.ethash_search(None, SEED, n_items, header, 1 << 33, grid * share, eth_target))
         assert 0 < want_e[0] <= 64
         rb, rs, re_ = H.new_search_results(), H.new_search_results(), H.new_search_results()
-        plan.launch_n([H.blake2b_args(rb, count, 0xFFFFF000, EASY10), H.sha256d_args(rs, count, 17), H.ethash_args(re_, 1 << 33)],
-                      grid_blocks=grid)
+        by_kernel = [H.blake2b_args(rb, count, 0xFFFFF000, EASY10), H.sha256d_args(rs, count, 17), H.ethash_args(re_, 1 << 33)]
+        plan.launch_n([by_kernel[k] for k in order], grid_blocks=grid)
         sync()
-        assert H.read_search_results(rb) == want_b, preset
-        assert H.read_search_results(rs) == want_s, preset
-        assert H.read_search_results(re_) == want_e, preset
+        assert H.read_search_results(rb) == want_b, (preset, order)
+        assert H.read_search_results(rs) == want_s, (preset, order)
+        assert H.read_search_results(re_) == want_e, (preset, order)
+    with pytest.raises(H.HfuseError) as e:          # three kernels that are none of the built lists: said when the plan is made
+        H.Config("- File: x\n  Kernels: [blake2b_gpu_hash, sia_blake2b_gpu_hash, ethash_search]\n", kernels_yaml).plan(0)
+    assert e.value.code == L.HF_EUNSUPPORTED
 
 
 def _strict(found_hits, limit, key):

@@ -3,6 +3,8 @@ Bit-exact against the oracle / PyTorch CPU ops for im2col, max_pool (values and
 int64 argmax), upsample and histogram counts; 1e-5 relative for batch-norm
 mean / invstd (tolerance of the fp32 Welford tree against the fp64 two-pass)."""
 import numpy as np
+import os
+
 import pytest
 import torch
 
@@ -456,28 +458,25 @@ def test_fused_histc_maxpool_full_benchmark_size(cuda, cfg):
 
 
 def test_bounded_builds_at_every_wave_count(cuda, cfg):
-    """The register-bounded builds of the shipped thread partitions -- at the occupancy formula's own value
-    (5, 6 and 7 waves per SIMD) and at 8 -- give the same bits as the plain build."""
+    """The register-bounded builds of the thread partitions -- the benchmarked pairs at each of 5, 6, 7 and 8 waves
+    per SIMD, three more shipped pairs at their formula's value and at 8 -- give the same bits as the plain build."""
     cases = [("im2col_kernel", "MaxPoolForward", lambda: Im2col(cuda, 4, 16, 56, 56),
-              lambda: MaxPool(cuda, 4, 16, 112, 112, (3, 3), (2, 2), (1, 1)), 5),
+              lambda: MaxPool(cuda, 4, 16, 112, 112, (3, 3), (2, 2), (1, 1)), (5, 6, 7, 8)),
              ("kernelHistogram1D", "MaxPoolForward", lambda: Histc(cuda, 1 << 20),
-              lambda: MaxPool(cuda, 4, 32, 64, 64, (2, 2), (2, 2), (0, 0)), 7),
+              lambda: MaxPool(cuda, 4, 32, 64, 64, (2, 2), (2, 2), (0, 0)), (5, 6, 7, 8)),
              ("batch_norm_collect_statistics_kernel", "upsample_nearest2d_out_frame", lambda: BnStats(cuda, 8, 32, 28, 28),
-              lambda: Upsample(cuda, 8, 16, 56, 56, (112, 112)), 8),
-             # the other shipped thread partitions whose formula gives fewer than 8
+              lambda: Upsample(cuda, 8, 16, 56, 56, (112, 112)), (5, 6, 7, 8)),
              ("im2col_kernel", "upsample_nearest2d_out_frame", lambda: Im2col(cuda, 4, 16, 56, 56),
-              lambda: Upsample(cuda, 8, 16, 56, 56, (112, 112)), 6),
-             ("im2col_kernel", "kernelHistogram1D", lambda: Im2col(cuda, 4, 16, 56, 56), lambda: Histc(cuda, 1 << 20), 7),
-             ("MaxPoolForward", "batch_norm_collect_statistics_kernel",
-              lambda: MaxPool(cuda, 4, 16, 112, 112, (3, 3), (2, 2), (1, 1)), lambda: BnStats(cuda, 8, 32, 28, 28), 7),
+              lambda: Upsample(cuda, 8, 16, 56, 56, (112, 112)), (6, 8)),
+             ("im2col_kernel", "kernelHistogram1D", lambda: Im2col(cuda, 4, 16, 56, 56), lambda: Histc(cuda, 1 << 20), (7, 8)),
              ("im2col_kernel", "upsample_bilinear2d_out_frame", lambda: Im2col(cuda, 4, 16, 56, 56),
-              lambda: Bilinear(cuda, 4, 16, 56, 56, (112, 112)), 6)]
-    for k1, k2, m1, m2, formula in cases:
-        plan = cfg.plan(cfg.find_fusion(k1, k2), "hfuse_lb")
-        assert plan.launch_waves == (formula, formula)
-        for waves in (0, 8, 1):
+              lambda: Bilinear(cuda, 4, 16, 56, 56, (112, 112)), (6, 8))]
+    for k1, k2, m1, m2, built in cases:
+        plan = cfg.plan(cfg.find_fusion(k1, k2), "hfuse", 0)       # the thread partition at the table's shape
+        plan.set_block(256, 256)
+        for waves in built:
             plan.set_launch_waves(waves)
-            assert plan.launch_waves[1] in (formula, 8)
+            assert plan.launch_waves[1] == waves
             a, b = m1(), m2()
             plan.launch(a.args, b.args)
             sync()
@@ -533,12 +532,43 @@ def test_three_kernel_fusions(cuda):
         c.check()
     with pytest.raises(H.HfuseError):
         plan.time_n(0, [[a.args, b.args, c.args]], 0, 1)
+    # the launch-bound presets of a three-kernel list run its build bounded for 8 waves per SIMD
+    assert t.plan(i, "hfuse_lb").launch_waves[1] == 8 and t.plan(i, "vfuse_lb").launch_waves[1] == 8 and t.plan(i).launch_waves[1] == 0
     # empty work in one part
     a, c = Im2col(cuda, 2, 3, 9, 10), BnStats(cuda, 4, 37, 6, 5)
     b = MaxPool(cuda, 2, 3, 9, 7, (2, 2), (2, 2), (0, 0))
     plan.launch_n([a.args, b.args, c.args], grid_blocks=1)
     sync()
     a.check(); b.check(); c.check()
+
+
+@pytest.mark.parametrize("order", [(2, 0, 1), (1, 2, 0), (2, 1, 0), (0, 2, 1)])
+def test_three_kernel_lists_in_any_order(cuda, order):
+    """The Context partitions a block among the kernels in the order the list names them
+    (include/KernelFusion.h:45-80): the reference's three-kernel lists with their kernels permuted run the same
+    instantiation with other thread bounds, the arguments following the list's order."""
+    import hfuse_amd
+    kernels = open(os.path.join(hfuse_amd.CONFIG_DIR, "gfx950_kernels.yaml")).read()
+    lists = [("im2col_kernel", "MaxPoolForward", "batch_norm_collect_statistics_kernel"),
+             ("MaxPoolForward", "kernelHistogram1D", "batch_norm_collect_statistics_kernel")]
+    make = {"im2col_kernel": lambda: Im2col(cuda, 4, 16, 24, 24),
+            "MaxPoolForward": lambda: MaxPool(cuda, 4, 16, 48, 48, (3, 3), (2, 2), (1, 1)),
+            "batch_norm_collect_statistics_kernel": lambda: BnStats(cuda, 4, 37, 6, 8),
+            "kernelHistogram1D": lambda: Histc(cuda, 300001)}
+    for names in lists:
+        listed = [names[k] for k in order]
+        text = "- File: permuted\n  Kernels:\n" + "".join(f"    - {k}\n" for k in listed) + "  Blocks: [128, 256, 192]\n"
+        cfg = H.Config(text, kernels)
+        for preset, grid in (("hfuse", 0), ("hfuse", 7), ("vfuse", 0), ("hfuse_lb", 0)):
+            plan = cfg.plan(0, preset)
+            q = plan.partition_n
+            if preset != "vfuse":
+                assert list(q.lo)[:3] == [0, 128, 384] and list(q.hi)[:3] == [128, 384, 576]
+            work = [make[k]() for k in listed]
+            plan.launch_n([w.args for w in work], grid_blocks=grid)
+            sync()
+            for w in work:
+                w.check()
 
 
 def test_time_pair_continues_the_rotation(cuda, cfg):

@@ -3,6 +3,8 @@ the oracle, and the error behaviour at the C-ABI."""
 import ctypes as C
 import re
 
+import os
+
 import pytest
 
 import hfuse_amd
@@ -135,8 +137,13 @@ def test_fusion_list_errors():
     with pytest.raises(hfuse_amd.HfuseError) as e:
         cfg.num_splits(0)
     assert e.value.code == L.HF_EUNSUPPORTED
+    with pytest.raises(hfuse_amd.HfuseError) as e:                      # three kernels that are none of the built lists:
+        cfg.plan(1)                                                     # said when the plan is made, not at the launch
+    assert e.value.code == L.HF_EUNSUPPORTED and "in any order" in e.value.message
+    too_wide = Config("- File: three\n  Kernels: [im2col_kernel, MaxPoolForward, batch_norm_collect_statistics_kernel]\n",
+                      KERNELS_MAP)
     with pytest.raises(hfuse_amd.HfuseError) as e:                      # 512 + 256 + 512 threads
-        cfg.plan(1)
+        too_wide.plan(0)
     assert e.value.code == L.HF_EINVAL and "exceeds 1024" in e.value.message
     assert cfg.num_splits(1) == 5                                        # the loop varies the first two: 128 .. 640 < 768
     cfg.plan(2)
@@ -282,7 +289,8 @@ def test_local_index_follows_the_remap(cfg):
 
 def test_barrier_policy(cfg):
     assert cfg.plan(0).partition.barrier_mode == L.HF_BARRIER_NONE
-    bn_up = cfg.plan(1)
+    # the policy of the library, whatever mode the shipped list tunes this pair to: an explicit split takes no tuned keys
+    bn_up = cfg.plan(1, "hfuse", 0)
     assert bn_up.partition.barrier_mode == L.HF_BARRIER_SUBSET
     with pytest.raises(hfuse_amd.HfuseError):
         bn_up.set_barrier_mode(L.HF_BARRIER_MATCHED)  # upsample never synchronises
@@ -531,46 +539,69 @@ def test_constants_objects_are_independent_of_the_process_wide_set(cfg):
         H.Constants().set_ethash(type("T", (), {"data_ptr": lambda self: 8})(), 4, bytes(32), 1)  # misaligned DAG
 
 
-def test_launch_bound_formula_and_built_variants(cfg):
+def test_launch_bound_formula_and_built_variants():
     """The register-cap axis: the occupancy formula of the reference's printer (KernelPrinter.cpp:44-66) with
-    this part's constants, hand-worked for the five benchmarked pairs of the shipped list, and the build each
-    request resolves to.  im2col(Reg 42, 256 thr) + max-pool(32, 448): min(131072/42/256 = 12, 131072/32/448 = 9,
-    2048/704 = 2) = 2 blocks of 704 threads = 5 waves per SIMD; bn(23,128) + upsample(22,128): min(44, 46, 8) = 8
-    blocks of 256 = 8; histogram(19,768) + max-pool(32,128): min(8, 32, 2) = 2 of 896 = 7; SHA-256d(70,128) +
-    Blake2b(76,128): min(14, 13, 8) = 8 of 256 = 8; Ethash(116,128) + Blake2b(76,64): min(8, 26, 10) = 8 of 192 = 6."""
-    want = [5, 8, 7, 8, 6]
-    for i, w in enumerate(want):
+    this part's constants (128 K registers, 2048 threads a CU), hand-worked for the five benchmarked pairs at fixed
+    block shapes, and the build each request resolves to.  B blocks of T threads are B * T / 64 waves on four SIMDs:
+    the bound is rounded up, so that all of them fit.
+      im2col(Reg 42, 256 thr) + max-pool(32, 448): min(131072/42/256 = 12, 131072/32/448 = 9, 2048/704 = 2) = 2 blocks
+        of 704 threads = 22 waves = 5.5 -> 6 waves per SIMD;
+      bn(23, 128) + upsample(22, 128): min(44, 46, 8) = 8 blocks of 256 = 32 waves -> 8;
+      histogram(19, 768) + max-pool(32, 128): min(8, 32, 2) = 2 of 896 = 28 waves -> 7;
+      SHA-256d(70, 128) + Blake2b(76, 128): min(14, 13, 8) = 8 of 256 -> 8;
+      Ethash(116, 128) + Blake2b(76, 64): min(8, 26, 10) = 8 of 192 = 24 waves -> 6;
+      max-pool(32, 64) + bn(23, 128): min(64, 44, 10) = 10 of 192 = 30 waves = 7.5 -> 8."""
+    kernels = open(os.path.join(hfuse_amd.CONFIG_DIR, "gfx950_kernels.yaml")).read()
+    shapes = [("im2col_kernel", "MaxPoolForward", 256, 448, 6),
+              ("batch_norm_collect_statistics_kernel", "upsample_nearest2d_out_frame", 128, 128, 8),
+              ("kernelHistogram1D", "MaxPoolForward", 768, 128, 7),
+              ("sha256d_gpu_hash_shared", "sia_blake2b_gpu_hash", 128, 128, 8),
+              ("ethash_search", "sia_blake2b_gpu_hash", 128, 64, 6),
+              ("MaxPoolForward", "batch_norm_collect_statistics_kernel", 64, 128, 8)]
+    text = "".join(f"- File: f{n}\n  Kernels: [{a}, {b}]\n  Split: {t1}\n  Threads: {t1 + t2}\n" for n, (a, b, t1, t2, _) in enumerate(shapes))
+    cfg = Config(text, kernels)
+    for i, (_, _, t1, t2, w) in enumerate(shapes):
         plain, lb = cfg.plan(i), cfg.plan(i, "hfuse_lb")
         assert plain.launch_waves == (w, 0), (i, plain.launch_waves)      # the plain preset runs the plain build
-        assert lb.launch_waves == (w, w), (i, lb.launch_waves)            # the _lb preset the pair's own bounded build
-        assert lb.partition.launch_blocks * lb.partition.launch_threads // 256 == w
+        assert lb.launch_waves == (w, w), (i, lb.launch_waves)            # the _lb preset the build bounded at the formula's value
+        blocks, threads = lb.partition.launch_blocks, lb.partition.launch_threads
+        assert threads == t1 + t2 and -(-blocks * (threads // 64) // 4) == w
         plain.set_launch_bound(True)
         assert plain.launch_waves == (w, w)
         plain.set_launch_waves(8)
         assert plain.launch_waves == (w, 8)
-        plain.set_launch_waves(3)                                         # below the pair's own value: its own build, else 8
-        assert plain.launch_waves == (w, w if w < 8 else 8)
+        with pytest.raises(hfuse_amd.HfuseError):
+            plain.set_launch_waves(9)
+        if i < 5:
+            # the five benchmarked pairs are built at 5, 6, 7 and 8 waves per SIMD: any request gets the smallest
+            # build that is not below it (up to four the plain build's launch bound already holds)
+            for ask, got in ((7, 7), (6, 6), (5, 5), (3, 5), (1, 5)):
+                plain.set_launch_waves(ask)
+                assert plain.launch_waves == (w, got), (i, ask, plain.launch_waves)
+            # ... so another block shape of the pair runs the build at its own formula value
+            other = cfg.plan(i, "hfuse_lb")
+            other.set_block(64, 64)
+            f, b = other.launch_waves
+            assert f == b and 5 <= f <= 8
+        else:
+            plain.set_launch_waves(3)                                     # every other pair: the 8-wave build
+            assert plain.launch_waves == (w, 8)
         plain.set_launch_waves(0)
         plain.set_launch_bound(False)
         assert plain.launch_waves == (w, 0)
-        with pytest.raises(hfuse_amd.HfuseError):
-            plain.set_launch_waves(9)
         plain.set_barrier_mode(L.HF_BARRIER_BLOCKIDX)
         plain.set_launch_bound(True)
         assert plain.launch_waves[1] == 0                                 # the block-index partition has no bounded build
-    # beyond the benchmarked five: the shipped thread partitions whose formula gives fewer than 8 waves have a build at
-    # that value too -- im2col(42, 256) + upsample(22, 512): min(12, 11, 2) = 2 blocks of 768 threads = 6 waves per SIMD
+    # three more pairs of the shipped list have a second build at the formula's value of their shipped shape --
+    # im2col(42, 256) + upsample(22, 512): min(12, 11, 2) = 2 blocks of 768 threads = 6 waves per SIMD;
+    # im2col(42, 256) + histogram(19, 640): min(12, 10, 2) = 2 of 896 = 7; im2col + bilinear upsampling (32, 512): 6
+    shipped = hfuse_amd.default_config()
     for k1, k2, w in (("im2col_kernel", "upsample_nearest2d_out_frame", 6), ("im2col_kernel", "kernelHistogram1D", 7),
-                      ("MaxPoolForward", "batch_norm_collect_statistics_kernel", 7),
                       ("im2col_kernel", "upsample_bilinear2d_out_frame", 6)):
-        p = cfg.plan(cfg.find_fusion(k1, k2), "hfuse_lb")
+        p = shipped.plan(shipped.find_fusion(k1, k2), "hfuse_lb")
         assert p.launch_waves == (w, w), (k1, k2, p.launch_waves)
         p.set_launch_waves(8)
         assert p.launch_waves == (w, 8)
-    # every other pair has the 8-wave build only
-    p = cfg.plan(cfg.find_fusion("upsample_nearest2d_out_frame", "batch_norm_collect_statistics_kernel"), "hfuse_lb")
-    p.set_launch_waves(3)
-    assert p.launch_waves[1] == 8
 
 
 TRIPLE_TABLE = """
