@@ -50,10 +50,10 @@ TRAFFIC_BYTES = {"bn_upsample": 156.54e6, "im2col_maxpool": 443.27e6, "histc_max
 OPS_SHA256D = 4336
 OPS_BLAKE2B = 2528
 ETHASH_BYTES = 8192               # 64 accesses x 128 bytes of DAG per hash
-# VALU instructions a wavefront issues per hash (SQ_INSTS_VALU of the native kernels over 2^24 hashes, x 64 lanes / 2^24:
-# profiles/all_pairs_sq_counters.md) and the rate one CU issues them at: 64 lanes per clock
-VALU_INSTS_SHA256D = 3082
-VALU_INSTS_BLAKE2B = 1101
+# VALU instructions a wavefront issues per hash (SQ_INSTS_VALU of the native kernels over their 2^30 nonces, x 64 lanes /
+# 2^30: profiles/hash_kernels_valu_issue.md) and the rate one CU issues them at: 64 lanes per clock
+VALU_INSTS_SHA256D = 3029
+VALU_INSTS_BLAKE2B = 1751
 VALU_ISSUE_GLANES = 256 * 64 * 2.4  # 256 CUs x 64 lanes x 2.4 GHz, in G lane-instructions/s
 
 # What a fused tensor pair could reach at best: its bytes at the rates the library's bare stream kernels reach on

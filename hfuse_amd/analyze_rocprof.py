@@ -11,7 +11,7 @@ block shape instead:
 
     native_kernel<XBody, ...>            ST   one original kernel (native_kernel_capped: the same with its
                                               residency capped, as im2col is launched)
-    vertical_kernel<XBody, YBody, ...>   VF   the same threads run both bodies
+    vertical_kernel<XBody, YBody, ...>   VF   the same threads run both bodies, tagged with the workgroup size
     fused_kernel<XBody, YBody, .., 0>    HF   horizontally fused, tagged with the workgroup size
     fused_kernel<XBody, YBody, .., 1>    HF+M the same with the shared hardware barrier
     blockidx_kernel<XBody, YBody, ...>   BI   block-index partition
@@ -70,7 +70,7 @@ class KernelKey:
     block: int                     # workgroup size of the launch
 
     def label(self) -> str:
-        return self.tag if self.tag in ("ST", "VF", "VF-LB") else f"{self.tag}@{self.block}"
+        return self.tag if self.tag == "ST" else f"{self.tag}@{self.block}"
 
 
 def parse_kernel_name(name: str) -> Optional[Tuple[str, Tuple[str, ...]]]:
@@ -91,7 +91,7 @@ def parse_kernel_name(name: str) -> Optional[Tuple[str, Tuple[str, ...]]]:
         return "VF" + lb, tuple(bodies)
     if kind == "blockidx_kernel":
         return "BI", tuple(bodies)
-    matched = params.rstrip().endswith("true")
+    matched = re.search(r",\s*true\b", params) is not None   # fused_kernel<K1, K2, T, MATCHED> / fused_kernel_lb<..., MATCHED, W>
     return ("HF+M" if matched else "HF") + lb, tuple(bodies)
 
 

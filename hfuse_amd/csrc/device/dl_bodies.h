@@ -15,7 +15,7 @@
 namespace hfuse {
 
 // Hints (0 always means the general path).
-enum { HINT_GENERIC = 0, HINT_IM2COL_3X3_S1P1 = 1, HINT_POOL_K3S2P1 = 1, HINT_POOL_K2S2P0 = 2, HINT_UP_2X = 1, HINT_BN_VEC4 = 1, HINT_HIST_VEC4 = 1, HINT_HIST_POW2 = 2, HINT_HIST_GLOBAL = 8 /* more bins than the LDS budget: count straight into global memory */, HINT_HIST_HEAD_SHIFT = 4 /* bits 4-5: elements before the first 16-byte boundary */, HINT_BILINEAR_VEC4 = 1, HINT_BILINEAR_2X = 2,
+enum { HINT_GENERIC = 0, HINT_IM2COL_3X3_S1P1 = 1, HINT_POOL_K3S2P1 = 1, HINT_POOL_K2S2P0 = 2, HINT_UP_2X = 1, HINT_BN_VEC4 = 1, HINT_HIST_VEC4 = 1, HINT_HIST_POW2 = 2, HINT_HIST_GLOBAL = 8 /* more bins than the LDS budget: count straight into global memory */, HINT_HIST_HEAD_SHIFT = 4 /* bits 4-5: elements before the first 16-byte boundary */, HINT_BILINEAR_VEC4 = 1, HINT_BILINEAR_2X = 2, HINT_BILINEAR_2X_ALIGN = 3,
        // general path with 32-bit index arithmetic: every tensor of the call has fewer than 2^31 elements
        HINT_IDX32 = 0x100 };
 
@@ -236,7 +236,9 @@ struct MaxPoolBody {
     const unsigned ph2 = PW >> 1;
     const unsigned n2 = (unsigned)a.nthreads >> 1;
     const unsigned stride = sb.gstride();
-    for (unsigned idx2 = sb.gtid(); idx2 < n2; idx2 += stride) {
+    // One work item: its K window rows are loaded first (`load_item`), compared and stored later (`finish_item`), so
+    // that a thread which loops over several items has the loads of two of them in flight at a time.
+    auto load_item = [&](unsigned idx2, f32x4 (&v)[K], float (&left)[K]) __attribute__((always_inline)) {
       const unsigned pw2 = idx2 % ph2;
       const unsigned t = idx2 / ph2;
       const unsigned ph = t % PH;
@@ -244,18 +246,7 @@ struct MaxPoolBody {
       const float *plane = a.bottom_data + (size_t)nc * H * W;
       const int hstart = (int)ph * 2 - P;
       const unsigned wbase = pw2 << 2;
-      float maxv[2];
-      int maxi[2];
       const int h0 = hstart < 0 ? 0 : hstart;
-#pragma unroll
-      for (int o = 0; o < 2; o++) {
-        const int ws = (int)wbase + 2 * o - P;
-        maxv[o] = -INFINITY;
-        maxi[o] = h0 * (int)W + (ws < 0 ? 0 : ws);
-      }
-      // issue every row's loads before the compare chain
-      f32x4 v[K];
-      float left[K];
 #pragma unroll
       for (int i = 0; i < K; i++) {
         const int h = hstart + i;
@@ -284,6 +275,21 @@ struct MaxPoolBody {
           const float from_left = dpp_f32<0x138>(v[i].w);
           if (sb.lane() != 0) left[i] = from_left;
         }
+      }
+    };
+    auto finish_item = [&](unsigned idx2, const f32x4 (&v)[K], const float (&left)[K]) __attribute__((always_inline)) {
+      const unsigned pw2 = idx2 % ph2;
+      const unsigned ph = (idx2 / ph2) % PH;
+      const int hstart = (int)ph * 2 - P;
+      const unsigned wbase = pw2 << 2;
+      const int h0 = hstart < 0 ? 0 : hstart;
+      float maxv[2];
+      int maxi[2];
+#pragma unroll
+      for (int o = 0; o < 2; o++) {
+        const int ws = (int)wbase + 2 * o - P;
+        maxv[o] = -INFINITY;
+        maxi[o] = h0 * (int)W + (ws < 0 ? 0 : ws);
       }
 #pragma unroll
       for (int i = 0; i < K; i++) {
@@ -314,7 +320,7 @@ struct MaxPoolBody {
       const i64x2 om = {maxi[0], maxi[1]};
       f32x2 *vp = reinterpret_cast<f32x2 *>(a.top_data + (size_t)idx2 * 2);
       i64x2 *mp = reinterpret_cast<i64x2 *>(a.top_mask + (size_t)idx2 * 2);
-      if ((HF_TAKEAPART & 1) && K == 2 && !(maxv[0] == 12345.678f && maxi[1] == -7)) continue;  // keeps the loads alive
+      if ((HF_TAKEAPART & 1) && K == 2 && !(maxv[0] == 12345.678f && maxi[1] == -7)) return;  // keeps the loads alive
 #if HF_NT_STORES
       __builtin_nontemporal_store(ov, vp);
       __builtin_nontemporal_store(om, mp);
@@ -322,6 +328,19 @@ struct MaxPoolBody {
       *vp = ov;
       *mp = om;
 #endif
+    };
+    // Two items per trip (the second one `stride` further on; the lanes that have one are a prefix of the wave, so
+    // every lane that shifts a halo column in still has its left neighbour).  A launch in which every thread
+    // has one item -- the native one -- never enters the second half.
+    for (unsigned idx2 = sb.gtid(); idx2 < n2; idx2 += 2 * stride) {
+      const unsigned idx_b = idx2 + stride;
+      const bool has_b = idx_b < n2;
+      f32x4 va[K], vb[K];
+      float la[K], lb[K];
+      load_item(idx2, va, la);
+      if (has_b) load_item(idx_b, vb, lb);
+      finish_item(idx2, va, la);
+      if (has_b) finish_item(idx_b, vb, lb);
     }
   }
 };
@@ -504,6 +523,78 @@ struct UpsampleBilinearBody {
     }
   }
 
+  // The same work-item shape for align_corners = true at twice the size.  There src = dst * (in - 1) / (out - 1)
+  // drifts from dst / 2 - 1/2 to dst / 2 across the image, so which two of the four window columns 2q-1..2q+2 (and
+  // which two of the three rows j-1..j+1) an output blends differs from output to output: the index is computed
+  // per output with the general path's expressions and selects among the values the work item already holds in
+  // registers.  The host takes this path only after checking, with the same fp32 steps, that every output's
+  // sources lie inside its work item's window.
+  template <class SB>
+  static __device__ __forceinline__ void exact2x_align(const Args &a, SB &sb) {
+    const unsigned H1 = (unsigned)a.idata.sizes[2], W1 = (unsigned)a.idata.sizes[3];
+    const unsigned W2 = W1 * 2u;
+    const unsigned wq = W1 >> 1;
+    const unsigned NC = (unsigned)(a.idata.sizes[0] * a.idata.sizes[1]);
+    const unsigned n = NC * H1 * wq;
+    const unsigned stride = sb.gstride();
+    const unsigned lane = sb.lane();
+    auto pick4 = [](const float (&w)[4], int i) { return i <= 0 ? w[0] : i == 1 ? w[1] : i == 2 ? w[2] : w[3]; };
+    for (unsigned first = sb.gtid() - lane; first < n; first += stride) {
+      const bool valid = first + lane < n;
+      const unsigned idx = valid ? first + lane : n - 1;
+      const unsigned q = idx % wq;
+      const unsigned t = idx / wq;
+      const unsigned j = t % H1;
+      const unsigned nc = t / H1;
+      const float *pl = a.idata.data + (size_t)nc * H1 * W1 + 2u * q;
+      const unsigned jr[3] = {j > 0 ? j - 1 : 0u, j, j + 1 < H1 ? j + 1 : j};
+      const bool has_left = q > 0, has_right = q + 1 < wq;
+      float wl[4], wr[4];  // weight of the left / right source column of output 4q+k
+      int ci[4], cn[4];    // their positions in the window of columns 2q-1..2q+2
+#pragma unroll
+      for (int k = 0; k < 4; k++) {
+        const float w1r = src_index(a.rwidth, (int)(4u * q) + k, true);
+        const int x1 = (int)w1r;
+        wr[k] = rn_sub(w1r, (float)x1);
+        wl[k] = rn_sub(1.0f, wr[k]);
+        ci[k] = x1 + 1 - (int)(2u * q);
+        cn[k] = ci[k] + (x1 < (int)W1 - 1 ? 1 : 0);
+      }
+      float hl[3][4];  // horizontally interpolated rows j-1, j, j+1
+#pragma unroll
+      for (int r = 0; r < 3; r++) {
+        const float *row = pl + (size_t)jr[r] * W1;
+        const float2 m = *reinterpret_cast<const float2 *>(row);
+        float left = dpp_f32<0x138>(m.y);   // wave_shr:1 -- lane-1's second column
+        float right = dpp_f32<0x130>(m.x);  // wave_shl:1 -- lane+1's first column
+        if (lane == 0 && has_left) left = row[-1];
+        if (lane == 63 && has_right) right = row[2];
+        const float win[4] = {left, m.x, m.y, right};   // the outer two are never selected where the image ends
+#pragma unroll
+        for (int k = 0; k < 4; k++) hl[r][k] = rn_add(rn_mul(wl[k], pick4(win, ci[k])), rn_mul(wr[k], pick4(win, cn[k])));
+      }
+      float o[2][4];
+#pragma unroll
+      for (int s = 0; s < 2; s++) {
+        const float h1r = src_index(a.rheight, (int)(2u * j) + s, true);
+        const int y1 = (int)h1r;
+        const float h1l = rn_sub(h1r, (float)y1), h0l = rn_sub(1.0f, h1l);
+        const int ri = y1 + 1 - (int)j, rn = ri + (y1 < (int)H1 - 1 ? 1 : 0);   // positions among the rows j-1, j, j+1
+#pragma unroll
+        for (int k = 0; k < 4; k++) {
+          const float top = ri <= 0 ? hl[0][k] : ri == 1 ? hl[1][k] : hl[2][k];
+          const float bot = rn <= 0 ? hl[0][k] : rn == 1 ? hl[1][k] : hl[2][k];
+          o[s][k] = rn_add(rn_mul(h0l, top), rn_mul(h1l, bot));
+        }
+      }
+      if (valid) {
+        float *out = a.odata.data + ((size_t)nc * (2u * H1) + 2u * j) * W2 + 4u * q;
+        st4(out, f32x4{o[0][0], o[0][1], o[0][2], o[0][3]});
+        st4(out + W2, f32x4{o[1][0], o[1][1], o[1][2], o[1][3]});
+      }
+    }
+  }
+
   template <class SB>
   static __device__ __forceinline__ void run(const Args &a, SB &sb, unsigned char *, unsigned hint) {
     const int H1 = (int)a.idata.sizes[2], W1 = (int)a.idata.sizes[3];
@@ -514,6 +605,10 @@ struct UpsampleBilinearBody {
     const bool same = H1 == H2 && W1 == W2;
     if (hint == HINT_BILINEAR_2X) {
       exact2x(a, sb);
+      return;
+    }
+    if (hint == HINT_BILINEAR_2X_ALIGN) {
+      exact2x_align(a, sb);
       return;
     }
     if (hint == HINT_BILINEAR_VEC4) {

@@ -25,7 +25,7 @@ def test_parse_kernel_name():
     assert A.parse_kernel_name(F.replace("fused_kernel<", "fused_kernel_lb<").format(a="HistcBody", b="MaxPoolBody", m="false"))[0] == "HF-LB"
     assert A.parse_kernel_name(F.replace("fused_kernel<", "fused_kernel_lb<").format(a="HistcBody", b="BnStatsBody", m="true"))[0] == "HF+M-LB"
     assert A.parse_kernel_name(V.replace("vertical_kernel<", "vertical_kernel_lb<").format(a="Im2colBody", b="MaxPoolBody")) == ("VF-LB", ("im2col_kernel", "MaxPoolForward"))
-    assert A.KernelKey("HF-LB", ("a", "b"), 512).label() == "HF-LB@512" and A.KernelKey("VF-LB", ("a", "b"), 512).label() == "VF-LB"
+    assert A.KernelKey("HF-LB", ("a", "b"), 512).label() == "HF-LB@512" and A.KernelKey("VF-LB", ("a", "b"), 512).label() == "VF-LB@512"
     assert A.parse_kernel_name("void at::native::vectorized_elementwise_kernel<4, Foo>(int)") is None
     assert A.parse_kernel_name("void hfuse::(anonymous namespace)::copy_f32_kernel(float const*, float*, unsigned long long)") is None
     # every body the library instantiates has a YAML name
@@ -71,7 +71,7 @@ def test_exec_time_table_assigns_shared_natives_by_order(tmp_path):
     assert t["Im2Col+Maxpool"]["Maxpool"] == pytest.approx(31.0)
     h = t["Hist+Maxpool"]
     assert h["ST"] == pytest.approx(59.0) and h["HF@896"] == pytest.approx(59.0) and h["HF@1024"] == pytest.approx(61.0)
-    assert h["VF"] == pytest.approx(64.0) and h["Maxpool"] == pytest.approx(12.0)
+    assert h["VF@512"] == pytest.approx(64.0) and h["Maxpool"] == pytest.approx(12.0)
     md = A.render_exec_table(t)
     assert "| Im2Col+Maxpool | 78.00 | * | 72.00 | * | * | HF@768 | +8.3 |" in md
     assert "| Hist+Maxpool | 59.00 | 64.00 | * | 59.00 | 61.00 | HF@896 | +0.0 |" in md

@@ -61,6 +61,7 @@ def test_valu_issue_rate_constants(bench):
     assert bench.VALU_ISSUE_GLANES == pytest.approx(39321.6)
     assert bench.VALU_PEAK_GOPS == 2 * bench.VALU_ISSUE_GLANES
     assert 0.95 < bench.VALU_INSTS_SHA256D * 12.9 / bench.VALU_ISSUE_GLANES < 1.05
+    assert 0.95 < bench.VALU_INSTS_BLAKE2B * 22.3 / bench.VALU_ISSUE_GLANES < 1.05     # Blake2b alone: 22.3 GH/s
 
 
 def test_roofline_constants(bench):
