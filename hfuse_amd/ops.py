@@ -208,11 +208,12 @@ def run(op: Op, stream=None):
     return op.outputs
 
 
-def run_fused(op1: Op, op2: Op, cfg: Optional[H.Config] = None, preset: str = "hfuse", stream=None):
+def run_fused(op1: Op, op2: Op, cfg: Optional[H.Config] = None, preset: str = "shipped", stream=None):
     """Launch the two ops as one fused kernel; returns (outputs of op1, outputs of op2).
 
     The pair is looked up in the fusion list of `cfg` (default: the shipped list) in either
-    order; a pair the list does not name raises KeyError."""
+    order; a pair the list does not name raises KeyError.  `preset`: one of the reference's four
+    (hfuse, hfuse_lb, vfuse, vfuse_lb) or "shipped", the form the list's entry was tuned to."""
     c = _config(cfg)
     try:
         first, second = op1, op2

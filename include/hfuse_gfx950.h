@@ -77,14 +77,27 @@ typedef struct {
  * and a string-keyed map of kernel rows.  `kernels_yaml` may also be the older
  * per-pair form, a bare sequence of rows (configs/im2col_maxpool.yaml); then
  * `fusion_yaml` may be NULL and the single fusion is that list in order.
- * Five keys beyond the reference's schema are accepted in a fusion entry
- * (the split tuner writes them): `Split: <threads>`, a tuned default for
- * kernel 1's share of the block, and `Threads: <threads>`, a tuned size of the
- * whole fused block (kernel 2 gets Threads - Split); both apply when a plan is
- * created with HF_SPLIT_TABLE.  `Lending: true|false` sets the plan's default
- * for hf_plan_set_lending and `Barrier: none|matched|subset|blockidx` the one
- * for hf_plan_set_barrier_mode (an illegal mode fails hf_plan_create);
- * `LaunchBound: true|false` the one for hf_plan_set_launch_bound.
+ * Block and flow sequences are both read (`Kernels: [a, b]`).
+ * Keys beyond the reference's schema are accepted in a fusion entry (the split
+ * tuner writes them); all of them apply to plans created with HF_SPLIT_TABLE and
+ * no explicit split_threads -- a plan of an explicit variant starts from the
+ * library's defaults:
+ *   `Split: <threads>`    kernel 1's share of the thread partition's block, and
+ *   `Threads: <threads>`  the size of that block (kernel 2 gets Threads - Split);
+ *   `Lending: true|false` the plan's default for hf_plan_set_lending;
+ *   `Barrier: none|matched|subset|blockidx` the one for hf_plan_set_barrier_mode
+ *                         (an illegal mode fails hf_plan_create);
+ *   `LaunchBound: true|false` the one for hf_plan_set_launch_bound;
+ *   `Preset: <preset>`    the preset the entry ships with, which a plan created
+ *                         with the preset "shipped" gets (the reference prints
+ *                         all four presets and the user keeps the fastest,
+ *                         main.cpp:182-193; without the key: hfuse);
+ *   `Blocks: [t1, t2]`    the threads that run each body under a vertical preset
+ *                         (for a three-kernel entry: the block shape, one count
+ *                         per kernel);
+ *   `Grids: [g1, g2]`     the workgroups each kernel of a pair strides over under
+ *                         the entry's own preset (hf_plan_set_grids; 0 = the
+ *                         library's choice).
  * A kernel row may carry one extra key, `NativeThreads: <threads>` (a multiple of 64, at most 1024): the
  * block the unfused kernel is launched with by hf_time_pair when that differs from BlockDim, which stays
  * the basis of the split enumeration (the histogram runs fastest alone at 768 threads, and BlockDim 768
@@ -138,7 +151,8 @@ enum {
 
 /*
  * Create a plan for fusion `fusion_index` of `cfg`.
- *   preset    : "hfuse" | "hfuse_lb" | "vfuse" | "vfuse_lb" (main.cpp:182-193).
+ *   preset    : "hfuse" | "hfuse_lb" | "vfuse" | "vfuse_lb" (main.cpp:182-193), or
+ *               "shipped": the one the entry's `Preset:` key names (hfuse without it).
  *               The hfuse presets partition the block's threads between the two
  *               kernels; the vfuse presets are the reference's baseline in which
  *               the same threads run kernel 1 and then kernel 2 (block =
@@ -163,11 +177,13 @@ HF_API void hf_plan_free(hf_plan *plan);
  */
 HF_API int hf_plan_set_barrier_mode(hf_plan *plan, int mode);
 /*
- * Per-half grids of the fused launch when the caller leaves grid_blocks <= 0:
- * half k strides over blocks [0, grid_k) and the launch covers max(grid1, grid2)
- * blocks.  0 keeps the library's choice for that half.  (The reference's halves
+ * Per-kernel grids of the fused launch when the caller leaves grid_blocks <= 0:
+ * kernel k strides over blocks [0, grid_k) and the launch covers max(grid1, grid2)
+ * blocks.  0 keeps the library's choice for that kernel.  (The reference's halves
  * share the launch grid; a half that wants fewer blocks simply ends early in
- * the surplus ones.)
+ * the surplus ones.)  Under a vertical preset this is how a few resident blocks
+ * take both kernels' work in turn: with grid_k = the number of CUs every block
+ * stays on its CU and its threads loop over kernel 1's work and then kernel 2's.
  */
 HF_API int hf_plan_set_grids(hf_plan *plan, int grid1, int grid2);
 /*
@@ -175,6 +191,9 @@ HF_API int hf_plan_set_grids(hf_plan *plan, int grid1, int grid2);
  * kernel 2 (multiples of 64, sum <= 1024), independent of the kernel table's
  * BlockDim, which stays the native launch shape.  The reference reaches the same
  * freedom through per-pair kernel tables (configs/im2col_maxpool.yaml ...).
+ * Under a vertical preset both bodies start at thread 0 (KernelFusion.h:76-78):
+ * the two counts are the threads that run each body (each <= 1024) and the block
+ * is the larger of them.
  */
 HF_API int hf_plan_set_block(hf_plan *plan, int threads1, int threads2);
 /*
@@ -191,14 +210,18 @@ HF_API int hf_plan_set_lending(hf_plan *plan, int on);
  * print `__launch_bounds__(T, B)` with B = min_k(regfile / Reg_k / size_k), capped by the
  * resident-thread limit (lib/KernelFuser/KernelPrinter.cpp:44-66), so that the compiler keeps
  * the fused kernel's registers within the occupancy the natives had.  On gfx950 that request
- * is a waves-per-SIMD bound, fixed at compile time: w = B * T / 256 with this part's 128 K
- * registers and 2048 resident threads per CU.  Every pair is built plain (bounded only by its
- * launch bound of 1024 or 512 threads) and register-bounded for 8 waves per SIMD (at most 64
- * vector registers, spilling to a private stack if it must); the benchmarked pairs whose formula
- * gives less than 8 have a second bounded build at exactly their value: im2col + max-pool 5,
- * histogram + max-pool 7, Ethash + Sia-Blake2b 6 (batch-norm + upsample and SHA-256d + Blake2b
- * come out at 8).  A request for w waves runs the pair's own build when w is at most its value
- * and the 8-wave build otherwise.
+ * is a waves-per-SIMD bound, fixed at compile time: w = ceil(B * T / 256) with this part's 128 K
+ * registers and 2048 resident threads per CU (B blocks of T threads are B * T / 64 waves on four
+ * SIMDs, and all of them have to fit).  Every pair is built plain (bounded only by its launch
+ * bound of 1024 or 512 threads, which holds four waves per SIMD) and register-bounded for 8 waves
+ * per SIMD (at most 64 vector registers, spilling to a private stack if it must).  The five
+ * benchmarked pairs (im2col + max-pool, batch-norm + upsample, histogram + max-pool, SHA-256d +
+ * Sia-Blake2b, Ethash + Sia-Blake2b) are built for each of 5, 6, 7 and 8 waves, so whatever block
+ * shape a plan of theirs has, a launch-bound preset runs the build bounded at exactly the
+ * formula's value; three more pairs of the shipped list have a second build at the value of
+ * their shipped shape (im2col + histogram 7, im2col + nearest / bilinear upsampling 6).  A
+ * request for w waves runs the smallest built bound that is not below w.  A three-kernel plan
+ * has the plain build and, for the launch-bound presets, one bounded for 8 waves.
  *   hf_plan_set_launch_bound: on = 1 / 0 run the bounded / the plain build whatever the preset;
  *                on < 0 by the preset (default): hfuse_lb and vfuse_lb run the bounded build when
  *                the formula asks for more than 4 waves per SIMD.
@@ -217,9 +240,12 @@ HF_API int hf_plan_partition(const hf_plan *plan, hf_partition *out);
  * Three-kernel fusions.  The reference's Context partitions one block among any number of kernels
  * (include/KernelFusion.h:45-80) and its lists name three in configs/crypt_four.yaml
  * (blake2b_gpu_hash, sha256d_gpu_hash_shared, ethash_search4), configs/im2col_maxpool_norm.yaml
- * and configs/maxpool_summary_norm.yaml; those three lists are built, in their listed order.
+ * and configs/maxpool_summary_norm.yaml; those three lists are built, and a list that names the
+ * same three kernels in another order runs the same instantiation with the thread bounds of its
+ * own order (any other three kernels: HF_EUNSUPPORTED from hf_plan_create).
  * hf_plan_create on such an entry gives a plan whose block is kernel 0's threads, then kernel
- * 1's, then kernel 2's (vfuse presets: all three start at thread 0 of a block of max threads).
+ * 1's, then kernel 2's, in the order the list names them (vfuse presets: all three start at thread
+ * 0 of a block of max threads); argument lists follow the list's order as well.
  *   split_idx     : as the reference's driver does it (main.cpp:215-227): only the first two
  *                   kernels' ExecTimes are varied, ExecTime_0 = 128*(idx+1), ExecTime_1 =
  *                   (d0 + d1) - ExecTime_0, the third keeps the table's (-1 without the key); the
