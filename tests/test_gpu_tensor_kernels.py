@@ -168,6 +168,23 @@ def test_maxpool(cuda, case):
     t.check()
 
 
+@pytest.mark.parametrize("case", [
+    (2, 3, 16, 24, (3, 3), (2, 2), (1, 1)),        # 3x3 / 2 / 1: two outputs per item
+    (3, 5, 18, 20, (2, 2), (2, 2), (0, 0)),        # 2x2 / 2: two outputs per item, two items in flight per trip
+    (1, 1, 2, 4, (2, 2), (2, 2), (0, 0)),          # a single item
+    (4, 7, 30, 62, (2, 2), (2, 2), (0, 0)),
+], ids=str)
+@pytest.mark.parametrize("grid,block", [(1, 64), (3, 128), (2, 1024), (61, 256)])
+def test_maxpool_on_fewer_threads_than_items(cuda, case, grid, block):
+    """A caller's small grid makes every thread loop over its items; odd and even trip counts, and threads whose
+    second item of a trip does not exist, give the same result as the one-item-per-thread launch."""
+    n, c, h, w, k, s, p = case
+    t = MaxPool(cuda, n, c, h, w, k, s, p, seed=grid + block)
+    H.launch_native("MaxPoolForward", t.args, grid, block)
+    sync()
+    t.check()
+
+
 def test_maxpool_dilated(cuda):
     t = MaxPool(cuda, 2, 2, 13, 11, (3, 2), (1, 2), (1, 1), (2, 1))
     H.launch_native("MaxPoolForward", t.args, grid_blocks=2, block_threads=64)
@@ -331,6 +348,26 @@ def test_histc_unaligned_input(cuda, offset, n):
     H.launch_native("kernelHistogram1D", H.histc_args(xd[offset:], out, 64, 0.0, 1.0))
     sync()
     assert np.array_equal(out.cpu().numpy(), O.histc(x[offset:].numpy(), 64, 0.0, 1.0))
+
+
+@pytest.mark.parametrize("block", [256, 1024])          # eight / four KiB-chunks in flight per wave
+@pytest.mark.parametrize("grid", [1, 3, 256])
+@pytest.mark.parametrize("n", [2047, 2048, 2049, 8191, 8192 * 5 + 3, 8192 * 4 * 7 + 4096 + 5])
+def test_histc_chunk_boundaries(cuda, n, grid, block):
+    """The input is read in per-wave chunks of four or eight KiB dealt over waves and workgroups; sizes one
+    element either side of a chunk, fewer chunks than waves and more chunks than one pass of the grid all count every
+    element once, with values outside the range (they go to a spare word of the table) mixed in."""
+    x = uniform((n + 1,), 77 + n, -0.25, 1.25)
+    x[::97] = float("nan")
+    x[5::131] = float("inf")
+    xd = x.to(cuda)
+    for off in (0, 1):
+        out = torch.zeros(100, device=cuda)
+        view = xd[off:off + n]
+        H.launch_native("kernelHistogram1D", H.histc_args(view, out, 100, 0.0, 1.0), grid, block)
+        sync()
+        want = O.histc(x[off:off + n].numpy(), 100, 0.0, 1.0)
+        assert np.array_equal(out.cpu().numpy(), want), (off, int(np.abs(out.cpu().numpy() - want).sum()))
 
 
 @pytest.mark.parametrize("nbins,lo,hi", [(1000, 0.0, 3.0), (7, -0.7, 0.0), (15360, 0.0, 10.0), (1024, 0.1, 0.9),

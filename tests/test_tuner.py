@@ -113,6 +113,37 @@ def test_launch_bound_key():
         plan.set_launch_bound(on)
 
 
+def test_vertical_candidates_and_their_keys():
+    """The vertical forms the tuner tries, and how a vertical winner is written next to the best thread partition."""
+    fusion, kernels = shipped()
+    cfg = H.Config(fusion, kernels)
+    i = cfg.find_fusion("kernelHistogram1D", "MaxPoolForward")
+    c = T.vertical_candidates(cfg, i, cus=256)
+    assert all(x.vertical and x.preset == "vfuse" and x.threads1 == x.threads2 for x in c)
+    assert {x.threads1 for x in c} == {512, 768, 1024}
+    assert T.Candidate(1024, 1024, grids=(0, 256), preset="vfuse") in c      # histogram on its own grid, pooling on resident blocks
+    assert T.Candidate(1024, 1024, grids=(512, 512), preset="vfuse") in c and T.Candidate(512, 512, preset="vfuse") in c
+    assert not any(x.threads1 == 768 and x.grids == (0, 0) and x.bounded for x in c)
+    # batch norm's blocks are rows of eight: 768 and 1024 divide, and so does 512
+    k = cfg.find_fusion("batch_norm_collect_statistics_kernel", "upsample_nearest2d_out_frame")
+    assert {x.threads1 for x in T.vertical_candidates(cfg, k, cus=256)} == {512, 768, 1024}
+    base = "- File: a\n  Kernels:\n    - kernelHistogram1D\n    - MaxPoolForward\n"
+    win, part = T.Candidate(1024, 1024, grids=(0, 256), preset="vfuse"), T.Candidate(832, 192)
+    text = T.apply_to_fusion_yaml(base, {0: (win, part)})
+    assert text == base + "  Split: 832\n  Threads: 1024\n  Preset: vfuse\n  Blocks: [1024, 1024]\n  Grids: [0, 256]\n"
+    new = H.Config(text, kernels)
+    v = new.plan(0, "shipped").partition
+    assert v.name.decode().endswith("vfuse_block_1024_1024") and v.launch_threads == 1024
+    h = new.plan(0, "hfuse").partition
+    assert (list(h.hi), h.launch_threads) == ([832, 1024], 1024)
+    assert T.apply_to_fusion_yaml(text, {0: None}) == base
+    assert T.apply_to_fusion_yaml(text, {0: (win, part)}) == text
+    # a bounded vertical winner names the bounded preset
+    lb = T.apply_to_fusion_yaml(base, {0: (T.Candidate(512, 512, bounded=True, preset="vfuse"), None)})
+    assert lb == base + "  Preset: vfuse_lb\n  Blocks: [512, 512]\n"
+    assert H.Config(lb, kernels).plan(0, "shipped").partition.name.decode().endswith("vfuse_lb_block_512_512")
+
+
 @pytest.mark.gpu
 def test_small_sweep_and_tuned_launch(cuda):
     from test_gpu_tensor_kernels import Im2col, MaxPool, sync
