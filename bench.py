@@ -42,7 +42,7 @@ VALU_PEAK_GOPS = 256 * 128 * 2.4  # 256 CUs x 128 lanes x 2.4 GHz int32 op/s in 
 # HBM bytes per launch of each fused kernel from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE, each scaled by what
 # the same counter reads for the plain copy kernel (profiles/tensor_pairs_hbm_traffic.md,
 # profiles/search_pairs_hbm_traffic.md); None where no counter run covers the shape
-TRAFFIC_BYTES = {"bn_upsample": 156.54e6, "im2col_maxpool": 443.27e6, "histc_maxpool": 329.44e6,
+TRAFFIC_BYTES = {"bn_upsample": 157.21e6, "im2col_maxpool": 443.33e6, "histc_maxpool": 328.36e6,
                  # 2 x 67 042 986 KiB FETCH_SIZE per 2^24 hashes (8 183.9 B per hash), at the benchmark's 2^28
                  "ethash_blake2b": 2 * 67042985.9 * 1024 * 16}
 

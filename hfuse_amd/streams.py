@@ -23,7 +23,7 @@ MIB = 1 << 20
 READ_SHAPES = ((256, 256), (512, 256), (256, 512), (1024, 256), (2048, 256))
 WRITE_SHAPES = ((256, 256), (512, 256), (1024, 256), (4096, 256), (16384, 256), (131072, 256))   # the last: one store a thread
 LINES_SHAPES = ((8192, 128), (32768, 128), (8192, 256))
-COPY_SHAPES = ((1024, 256), (4096, 256), (16384, 256), (4096, 512))
+COPY_SHAPES = ((1024, 256), (4096, 256), (16384, 256), (4096, 512), (32768, 256), (16384, 512))   # the last two: one vector a thread
 
 
 def _time(pattern, src, dst, nbytes, src_stride, dst_stride, nbuf, grid, block, warmup, iters, rounds=3):
