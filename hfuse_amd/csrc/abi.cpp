@@ -386,26 +386,28 @@ int prepare_bilinear(const hf_upsample_bilinear_args &a, Prepared &p) {
                      a.odata.sizes[2] == 2 * a.idata.sizes[2] && a.odata.sizes[3] == 2 * a.idata.sizes[3] &&
                      a.idata.sizes[3] % 2 == 0 && ((uintptr_t)a.idata.data & 7) == 0 &&
                      a.odata.sizes[2] < (1 << 22) && a.odata.sizes[3] < (1 << 22);
-  // the same work-item shape with align_corners: src = dst * (in - 1) / (out - 1) has to stay inside the window of each
-  // work item -- output columns 4q..4q+3 blend input columns 2q-1..2q+2, output rows 2j, 2j+1 input rows j-1..j+1 --
-  // which is checked here with the kernel's own fp32 steps (one pass over the output's width and height)
+  // the same work-item shape with align_corners: there src = dst * (in - 1) / (out - 1) drifts from dst / 2 - 1/2 to
+  // dst / 2 across the image, and as long as its integer part is (dst - 1) >> 1 (0 for dst = 0), as it is without
+  // align_corners, every output blends the same rows and columns of its work item's window and only the weights differ.
+  // Checked here with the kernel's own fp32 steps, one pass over the output's width and height (rounding breaks the
+  // rule near the far edge of images a few thousand pixels wide; those take the gathered path).
   bool twice_align = fast && a.align_corners && a.odata.sizes[2] == 2 * a.idata.sizes[2] &&
                      a.odata.sizes[3] == 2 * a.idata.sizes[3] && a.idata.sizes[3] % 2 == 0 &&
                      ((uintptr_t)a.idata.data & 7) == 0 && a.odata.sizes[2] <= (1 << 16) && a.odata.sizes[3] <= (1 << 16);
   if (twice_align) {
-    auto inside = [](float scale, int64_t out_size, int64_t in_size, int per_item, int first) {
+    auto fixed_sources = [](float scale, int64_t out_size) {
       for (int64_t dst = 0; dst < out_size; dst++) {
         const volatile float src = scale * (float)dst;
-        const int64_t i1 = (int64_t)(float)src, lo = (dst / per_item) * (per_item / 2) - first;
-        const int64_t i2 = i1 + (i1 < in_size - 1 ? 1 : 0);
-        if (i1 < lo || i1 < 0 || i2 > lo + (per_item == 4 ? 3 : 2) || i2 > in_size - 1) return false;
+        if ((int64_t)(float)src != (dst ? (dst - 1) >> 1 : 0)) return false;
       }
       return true;
     };
-    twice_align = inside(a.rwidth, a.odata.sizes[3], a.idata.sizes[3], 4, 1) && inside(a.rheight, a.odata.sizes[2], a.idata.sizes[2], 2, 1);
+    twice_align = fixed_sources(a.rwidth, a.odata.sizes[3]) && fixed_sources(a.rheight, a.odata.sizes[2]);
   }
   p.hint = twice ? HINT_BILINEAR_2X : twice_align ? HINT_BILINEAR_2X_ALIGN : fast ? HINT_BILINEAR_VEC4 : HINT_GENERIC;
-  p.items = (twice || twice_align) ? (unsigned long long)total / 8 : fast ? (unsigned long long)total / 4 : (unsigned long long)total;
+  // exact 2x: one work item per two input rows and two input columns
+  const unsigned long long row_pairs = ((unsigned long long)a.idata.sizes[2] + 1) / 2;
+  p.items = (twice || twice_align) ? (unsigned long long)a.idata.sizes[0] * a.idata.sizes[1] * row_pairs * (a.idata.sizes[3] / 2) : fast ? (unsigned long long)total / 4 : (unsigned long long)total;
   p.idx32 = true;  // every bilinear path counts in 32 bits (tensors below 2^32 elements)
   return HF_OK;
 }

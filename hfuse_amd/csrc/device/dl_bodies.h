@@ -455,20 +455,24 @@ struct UpsampleBilinearBody {
     return rn_add(rn_mul(h0, top), rn_mul(h1, bot));
   }
 
-  // Exact 2x, align_corners off, contiguous NCHW, even input width.  A work item owns input
-  // row j, columns 2q and 2q+1 and writes output rows 2j and 2j+1, columns 4q..4q+3: those
-  // eight outputs read input rows j-1, j, j+1 (clamped) at columns 2q-1..2q+2.  Each row is
-  // one 8-byte load; the two outer columns are the neighbouring lanes' elements, moved with a
-  // wavefront-wide DPP shift (lanes 0 and 63 fetch theirs from memory).  Weights and source
-  // indices come from the same expressions as the general path, so the bits are the same.
-  // The trip count is wave-uniform so every lane's neighbour is live.
-  template <class SB>
+  // Exact 2x, contiguous NCHW, even input width.  A work item owns input rows 2p, 2p+1, columns 2q, 2q+1 and
+  // writes output rows 4p..4p+3, columns 4q..4q+3: those sixteen outputs read input rows 2p-1..2p+2 (clamped)
+  // at columns 2q-1..2q+2.  Each row is one 8-byte load; the two outer columns are the neighbouring lanes'
+  // elements, moved with a wavefront-wide DPP shift (lanes 0 and 63 fetch theirs from memory).  At twice the
+  // size the source of output d starts at input (d - 1) >> 1 (0 for d = 0), with or without align_corners, so
+  // which rows and columns an output blends is fixed and only the weights differ: without align_corners
+  // 0.5 * (d + 0.5) - 0.5 is exact and the weights are the constants 0.25 / 0.75 (1 / 0 at the clamped first
+  // column and row); with align_corners the weights come from the general path's expressions, and the host
+  // takes this path only after checking, in the same fp32 steps, that every output's source index is the one
+  // above.  Either way the bits are those of the general path.  The trip count is wave-uniform so every
+  // lane's neighbour is live.
+  template <bool ALIGN, class SB>
   static __device__ __forceinline__ void exact2x(const Args &a, SB &sb) {
     const unsigned H1 = (unsigned)a.idata.sizes[2], W1 = (unsigned)a.idata.sizes[3];
     const unsigned W2 = W1 * 2u;
-    const unsigned wq = W1 >> 1;
+    const unsigned wq = W1 >> 1, hp = (H1 + 1u) >> 1;
     const unsigned NC = (unsigned)(a.idata.sizes[0] * a.idata.sizes[1]);
-    const unsigned n = NC * H1 * wq;
+    const unsigned n = NC * hp * wq;
     const unsigned stride = sb.gstride();
     const unsigned lane = sb.lane();
     for (unsigned first = sb.gtid() - lane; first < n; first += stride) {
@@ -476,21 +480,27 @@ struct UpsampleBilinearBody {
       const unsigned idx = valid ? first + lane : n - 1;
       const unsigned q = idx % wq;
       const unsigned t = idx / wq;
-      const unsigned j = t % H1;
-      const unsigned nc = t / H1;
+      const unsigned p = t % hp;
+      const unsigned nc = t / hp;
+      const unsigned j0 = 2u * p;
+      const bool second = j0 + 1u < H1;  // an odd height leaves the last work item of a plane one input row
       const float *pl = a.idata.data + (size_t)nc * H1 * W1 + 2u * q;
-      const unsigned jr[3] = {j > 0 ? j - 1 : 0u, j, j + 1 < H1 ? j + 1 : j};
+      const unsigned jr[4] = {j0 > 0 ? j0 - 1 : 0u, j0, second ? j0 + 1 : j0, j0 + 2 < H1 ? j0 + 2 : H1 - 1};
       const bool has_left = q > 0, has_right = q + 1 < wq;
       float wl[4], wr[4];  // weight of the left / right source column of output 4q+k
 #pragma unroll
       for (int k = 0; k < 4; k++) {
-        const float w1r = src_index(a.rwidth, (int)(4u * q) + k, false);
-        wr[k] = rn_sub(w1r, (float)(int)w1r);
+        if (ALIGN) {
+          const float w1r = src_index(a.rwidth, (int)(4u * q) + k, true);
+          wr[k] = rn_sub(w1r, (float)(int)w1r);
+        } else {
+          wr[k] = (k & 1) ? 0.25f : (k == 0 && !has_left) ? 0.0f : 0.75f;
+        }
         wl[k] = rn_sub(1.0f, wr[k]);
       }
-      float hl[3][4];  // horizontally interpolated rows j-1, j, j+1
+      float hl[4][4];  // horizontally interpolated rows 2p-1 .. 2p+2
 #pragma unroll
-      for (int r = 0; r < 3; r++) {
+      for (int r = 0; r < 4; r++) {
         const float *row = pl + (size_t)jr[r] * W1;
         const float2 m = *reinterpret_cast<const float2 *>(row);
         float left = dpp_f32<0x138>(m.y);   // wave_shr:1 -- lane-1's second column
@@ -504,93 +514,27 @@ struct UpsampleBilinearBody {
         // output 4q+3: source columns (2q+1, 2q+2); the last column pairs with itself
         hl[r][3] = rn_add(rn_mul(wl[3], m.y), rn_mul(wr[3], has_right ? right : m.y));
       }
-      // output row 2j blends rows (j-1, j), or (0, 1) with weights (1, 0) at the top edge;
-      // output row 2j+1 blends rows (j, j+1), the last row with itself
-      const float s0 = src_index(a.rheight, (int)(2u * j), false), s1 = src_index(a.rheight, (int)(2u * j) + 1, false);
-      const float b0 = rn_sub(s0, (float)(int)s0), t0 = rn_sub(1.0f, b0);
-      const float b1 = rn_sub(s1, (float)(int)s1), t1 = rn_sub(1.0f, b1);
-      float o0[4], o1[4];
+      // Output row 2j blends input rows (j-1, j), or (0, 1) with weights (1, 0) at the top edge; output row 2j+1
+      // blends (j, j+1), the last row with itself.  hl[0..3] are rows 2p-1, 2p, 2p+1, 2p+2, clamped to the plane.
+      float *out = a.odata.data + ((size_t)nc * (2u * H1) + 2u * j0) * W2 + 4u * q;
 #pragma unroll
-      for (int k = 0; k < 4; k++) {
-        o0[k] = rn_add(rn_mul(t0, hl[0][k]), rn_mul(b0, j > 0 ? hl[1][k] : hl[2][k]));
-        o1[k] = rn_add(rn_mul(t1, hl[1][k]), rn_mul(b1, hl[2][k]));
-      }
-      if (valid) {
-        float *out = a.odata.data + ((size_t)nc * (2u * H1) + 2u * j) * W2 + 4u * q;
-        st4(out, f32x4{o0[0], o0[1], o0[2], o0[3]});
-        st4(out + W2, f32x4{o1[0], o1[1], o1[2], o1[3]});
-      }
-    }
-  }
-
-  // The same work-item shape for align_corners = true at twice the size.  There src = dst * (in - 1) / (out - 1)
-  // drifts from dst / 2 - 1/2 to dst / 2 across the image, so which two of the four window columns 2q-1..2q+2 (and
-  // which two of the three rows j-1..j+1) an output blends differs from output to output: the index is computed
-  // per output with the general path's expressions and selects among the values the work item already holds in
-  // registers.  The host takes this path only after checking, with the same fp32 steps, that every output's
-  // sources lie inside its work item's window.
-  template <class SB>
-  static __device__ __forceinline__ void exact2x_align(const Args &a, SB &sb) {
-    const unsigned H1 = (unsigned)a.idata.sizes[2], W1 = (unsigned)a.idata.sizes[3];
-    const unsigned W2 = W1 * 2u;
-    const unsigned wq = W1 >> 1;
-    const unsigned NC = (unsigned)(a.idata.sizes[0] * a.idata.sizes[1]);
-    const unsigned n = NC * H1 * wq;
-    const unsigned stride = sb.gstride();
-    const unsigned lane = sb.lane();
-    auto pick4 = [](const float (&w)[4], int i) { return i <= 0 ? w[0] : i == 1 ? w[1] : i == 2 ? w[2] : w[3]; };
-    for (unsigned first = sb.gtid() - lane; first < n; first += stride) {
-      const bool valid = first + lane < n;
-      const unsigned idx = valid ? first + lane : n - 1;
-      const unsigned q = idx % wq;
-      const unsigned t = idx / wq;
-      const unsigned j = t % H1;
-      const unsigned nc = t / H1;
-      const float *pl = a.idata.data + (size_t)nc * H1 * W1 + 2u * q;
-      const unsigned jr[3] = {j > 0 ? j - 1 : 0u, j, j + 1 < H1 ? j + 1 : j};
-      const bool has_left = q > 0, has_right = q + 1 < wq;
-      float wl[4], wr[4];  // weight of the left / right source column of output 4q+k
-      int ci[4], cn[4];    // their positions in the window of columns 2q-1..2q+2
-#pragma unroll
-      for (int k = 0; k < 4; k++) {
-        const float w1r = src_index(a.rwidth, (int)(4u * q) + k, true);
-        const int x1 = (int)w1r;
-        wr[k] = rn_sub(w1r, (float)x1);
-        wl[k] = rn_sub(1.0f, wr[k]);
-        ci[k] = x1 + 1 - (int)(2u * q);
-        cn[k] = ci[k] + (x1 < (int)W1 - 1 ? 1 : 0);
-      }
-      float hl[3][4];  // horizontally interpolated rows j-1, j, j+1
-#pragma unroll
-      for (int r = 0; r < 3; r++) {
-        const float *row = pl + (size_t)jr[r] * W1;
-        const float2 m = *reinterpret_cast<const float2 *>(row);
-        float left = dpp_f32<0x138>(m.y);   // wave_shr:1 -- lane-1's second column
-        float right = dpp_f32<0x130>(m.x);  // wave_shl:1 -- lane+1's first column
-        if (lane == 0 && has_left) left = row[-1];
-        if (lane == 63 && has_right) right = row[2];
-        const float win[4] = {left, m.x, m.y, right};   // the outer two are never selected where the image ends
-#pragma unroll
-        for (int k = 0; k < 4; k++) hl[r][k] = rn_add(rn_mul(wl[k], pick4(win, ci[k])), rn_mul(wr[k], pick4(win, cn[k])));
-      }
-      float o[2][4];
-#pragma unroll
-      for (int s = 0; s < 2; s++) {
-        const float h1r = src_index(a.rheight, (int)(2u * j) + s, true);
-        const int y1 = (int)h1r;
-        const float h1l = rn_sub(h1r, (float)y1), h0l = rn_sub(1.0f, h1l);
-        const int ri = y1 + 1 - (int)j, rn = ri + (y1 < (int)H1 - 1 ? 1 : 0);   // positions among the rows j-1, j, j+1
+      for (int s = 0; s < 4; s++) {
+        float bw;
+        if (ALIGN) {
+          const float h1r = src_index(a.rheight, (int)(2u * j0) + s, true);
+          bw = rn_sub(h1r, (float)(int)h1r);
+        } else {
+          bw = (s & 1) ? 0.25f : (s == 0 && j0 == 0) ? 0.0f : 0.75f;
+        }
+        const float tw = rn_sub(1.0f, bw);
+        float o[4];
 #pragma unroll
         for (int k = 0; k < 4; k++) {
-          const float top = ri <= 0 ? hl[0][k] : ri == 1 ? hl[1][k] : hl[2][k];
-          const float bot = rn <= 0 ? hl[0][k] : rn == 1 ? hl[1][k] : hl[2][k];
-          o[s][k] = rn_add(rn_mul(h0l, top), rn_mul(h1l, bot));
+          const float top = s == 0 ? hl[0][k] : s == 3 ? hl[2][k] : hl[1][k];
+          const float bot = s == 0 ? (j0 > 0 ? hl[1][k] : hl[2][k]) : s == 3 ? hl[3][k] : hl[2][k];
+          o[k] = rn_add(rn_mul(tw, top), rn_mul(bw, bot));
         }
-      }
-      if (valid) {
-        float *out = a.odata.data + ((size_t)nc * (2u * H1) + 2u * j) * W2 + 4u * q;
-        st4(out, f32x4{o[0][0], o[0][1], o[0][2], o[0][3]});
-        st4(out + W2, f32x4{o[1][0], o[1][1], o[1][2], o[1][3]});
+        if (valid && (s < 2 || second)) st4(out + (size_t)s * W2, f32x4{o[0], o[1], o[2], o[3]});
       }
     }
   }
@@ -604,11 +548,11 @@ struct UpsampleBilinearBody {
     const bool align = a.align_corners != 0;
     const bool same = H1 == H2 && W1 == W2;
     if (hint == HINT_BILINEAR_2X) {
-      exact2x(a, sb);
+      exact2x<false>(a, sb);
       return;
     }
     if (hint == HINT_BILINEAR_2X_ALIGN) {
-      exact2x_align(a, sb);
+      exact2x<true>(a, sb);
       return;
     }
     if (hint == HINT_BILINEAR_VEC4) {

@@ -226,8 +226,11 @@ def test_upsample_nearest(cuda, shape, out):
                                        ((1, 5, 33, 200), (66, 400)), ((2, 2, 1, 64), (2, 128)),
                                        ((1, 1, 6, 8), (12, 24)), ((1, 1, 6, 8), (18, 16)),
                                        # more exact-2x shapes (with align_corners the sources drift by half a pixel across
-                                       # the image and every output selects its own two columns and rows of the work item's window)
+                                       # the image; the rows and columns an output blends stay those of align_corners off)
                                        ((1, 1, 2, 2), (4, 4)), ((2, 3, 9, 14), (18, 28)), ((1, 2, 64, 66), (128, 132)),
+                                       # two input rows per work item: one, two and three rows, wide and tall planes
+                                       ((2, 2, 2, 4), (4, 8)), ((1, 3, 3, 8), (6, 16)), ((1, 1, 2, 4096), (4, 8192)),
+                                       ((1, 1, 3001, 2), (6002, 4)), ((5, 1, 4, 2), (8, 4)),
                                        # four columns x four rows per work item: heights 1, 2, 3, 5, 13 leave partial row blocks
                                        ((3, 5, 7, 12), (13, 20)), ((2, 2, 3, 4), (1, 8)), ((1, 3, 2, 6), (2, 12)),
                                        ((1, 1, 4, 4), (3, 4)), ((2, 1, 9, 16), (5, 8)), ((4, 8, 28, 28), (56, 60))], ids=str)
