@@ -324,6 +324,9 @@ struct EthashBody {
 
   template <class SB>
   static __device__ __forceinline__ void run(const Args &a, SB &sb, unsigned char *, unsigned) {
+    // These waves spend most of their time waiting for DAG lines; whenever one of them can issue it goes first, and a
+    // partner's arithmetic fills the slots that are left (no effect natively, where every wave has this priority).
+    __builtin_amdgcn_s_setprio(3);
     const u32 gid = sb.bid * sb.nthreads + sb.tid;
     const u64 nonce = a.start_nonce + gid;
     const int lane_in_group = (int)(sb.tid & (kGroup - 1));
