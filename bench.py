@@ -130,6 +130,23 @@ def blockidx_plan(cfg, i):
     return plan
 
 
+def thread_partition_plan(cfg, i, bounded):
+    """The pair's thread partition at its tuned block shape, in the plain or the register-bounded build.  Where the
+    fusion list ships the pair as a block-index partition, the waves of one workgroup are still split between the
+    two kernels here, with the library's own barrier design and wave lending."""
+    import hfuse_amd
+    from hfuse_amd import _lib as L
+    plan = cfg.plan(i, "hfuse_lb" if bounded else "hfuse")
+    plan.set_launch_bound(bounded)
+    if plan.partition.barrier_mode == L.HF_BARRIER_BLOCKIDX:
+        plan.set_lending(True)
+        try:
+            plan.set_barrier_mode(L.HF_BARRIER_SUBSET)
+        except hfuse_amd.HfuseError:
+            plan.set_barrier_mode(L.HF_BARRIER_NONE)      # neither body synchronises
+    return plan
+
+
 def spread(samples):
     """{mode: [min, median, max]} of the per-launch milliseconds of every mode."""
     return {k: [min(v), statistics.median(v), max(v)] for k, v in samples.items()}
@@ -155,8 +172,9 @@ def judge(res):
     if "t_blockidx_ms" in res:
         ways["blockidx"] = res["t_blockidx_ms"]
     res["best_mode"] = min(ways, key=ways.get)
-    # modes within 0.3 % of the fastest run at the same speed for every practical purpose
-    res["modes_within_0p3pct_of_best"] = sorted(k for k, v in ways.items() if v <= ways[res["best_mode"]] * 1.003)
+    # The medians of one and the same form differ by up to half a percent from run to run (min_median_max_ms shows the
+    # spread inside a run): modes within 0.5 % of the fastest run at the same speed for every practical purpose.
+    res["modes_within_0p5pct_of_best"] = sorted(k for k, v in ways.items() if v <= ways[res["best_mode"]] * 1.005)
     res["hfuse_vs_vfuse_pct"] = (res["t_vfuse_ms"] / res["t_hfuse_ms"] - 1.0) * 100.0
     res["hfuse_vs_two_streams_pct"] = (res["t_two_streams_ms"] / res["t_hfuse_ms"] - 1.0) * 100.0
     res["hfuse_speedup_pct"] = (res["t_b2b_ms"] / res["t_hfuse_ms"] - 1.0) * 100.0
@@ -190,14 +208,10 @@ def time_tensor_pair(cfg, pair, rotations, sweep, fused_only, rounds=5):
     if not fused_only:
         runs = [("t_a_ms", plan, 0), ("t_b_ms", plan, 1), ("t_b2b_ms", plan, 2), ("t_fused_ms", plan, 3),
                 ("t_two_streams_ms", plan, 4)]                     # the launch pattern of the reference's own traces
-        def plain_partition():                 # the thread partition at its tuned shape, plain build
-            p = cfg.plan(i, "hfuse")
-            p.set_launch_bound(False)
-            return p
-        others = [("t_hfuse_ms", "hfuse", plain_partition),
+        others = [("t_hfuse_ms", "hfuse", lambda: thread_partition_plan(cfg, i, False)),
                   ("t_vfuse_ms", "vfuse", lambda: cfg.plan(i, "vfuse")),          # the reference's vertical baseline
                   ("t_blockidx_ms", "blockidx", lambda: blockidx_plan(cfg, i)),   # each workgroup runs one of the two kernels
-                  ("t_fused_lb_ms", "hfuse_lb", lambda: cfg.plan(i, "hfuse_lb"))] # the partition's register-bounded build
+                  ("t_fused_lb_ms", "hfuse_lb", lambda: thread_partition_plan(cfg, i, True))]
         for key, m, make in others:
             if m == mode and not sweep:
                 alias[key] = "t_fused_ms"       # the shipped form: one plan, one set of samples
@@ -215,7 +229,7 @@ def time_tensor_pair(cfg, pair, rotations, sweep, fused_only, rounds=5):
     res["min_median_max_ms"] = spread(samples)
     res["launches_per_sample"], res["rounds"], res["buffer_sets"] = per, rounds, nsets
     if not fused_only:
-        res["lb_waves_per_simd"] = cfg.plan(i, "hfuse_lb").launch_waves[1]
+        res["lb_waves_per_simd"] = thread_partition_plan(cfg, i, True).launch_waves[1]
     res["split"] = label
     res["shipped_mode"] = mode
     part = plan.partition
@@ -752,7 +766,7 @@ def main():
         "throughput": throughput,
         "pairs_at_least_10pct_faster": n_fast,
         "pairs_slower_than_back_to_back": sorted(n for n, r in report.items() if r.get("speedup_pct", 0.0) < 0.0),
-        "shipped_is_best_mode": {n: r.get("shipped_mode") in r.get("modes_within_0p3pct_of_best", [r.get("shipped_mode")])
+        "shipped_is_best_mode": {n: r.get("shipped_mode") in r.get("modes_within_0p5pct_of_best", [r.get("shipped_mode")])
                                  for n, r in report.items()},
         "stream_ceilings": ceilings,
         "roofline": roofline,

@@ -38,7 +38,7 @@ def test_judgement_of_a_pair(bench):
            "t_fused_ms": 0.0707, "t_hfuse_ms": 0.0707, "t_fused_lb_ms": 0.077}
     bench.judge(res)
     assert res["speedup_pct"] == pytest.approx((0.0785 / 0.0707 - 1) * 100)
-    assert res["best_mode"] == "hfuse" and res["modes_within_0p3pct_of_best"] == ["hfuse"]
+    assert res["best_mode"] == "hfuse" and res["modes_within_0p5pct_of_best"] == ["hfuse"]
     assert res["hfuse_vs_vfuse_pct"] == pytest.approx((0.075 / 0.0707 - 1) * 100)
     res.update(t_blockidx_ms=0.069)
     bench.judge(res)
@@ -47,9 +47,9 @@ def test_judgement_of_a_pair(bench):
     bench.judge(res)
     assert res["speedup_pct"] < 0 and res["best_mode"] == "blockidx"
     assert res["hfuse_speedup_pct"] == pytest.approx((0.0785 / 0.0707 - 1) * 100)
-    res.update(t_vfuse_ms=0.0691)        # within 0.3 % of the fastest: the same speed for every practical purpose
+    res.update(t_vfuse_ms=0.0692)        # within 0.5 % of the fastest: the same speed for every practical purpose
     bench.judge(res)
-    assert res["modes_within_0p3pct_of_best"] == ["blockidx", "vfuse"]
+    assert res["modes_within_0p5pct_of_best"] == ["blockidx", "vfuse"]
 
 
 def test_spread_of_samples(bench):
