@@ -40,6 +40,11 @@ __device__ __forceinline__ f32x4 ld4_stream(const float *p) {
 __device__ __forceinline__ size_t uniform_u64(size_t x) {
   return ((size_t)__builtin_amdgcn_readfirstlane((unsigned)(x >> 32)) << 32) | (unsigned)__builtin_amdgcn_readfirstlane((unsigned)x);
 }
+// Lane 63's value of a 64-bit quantity, as a wave-uniform value (every lane of the wavefront must be active).
+__device__ __forceinline__ size_t uniform_last_u64(size_t x) {
+  return ((size_t)(unsigned)__builtin_amdgcn_readlane((int)(unsigned)(x >> 32), 63) << 32) |
+         (unsigned)__builtin_amdgcn_readlane((int)(unsigned)x, 63);
+}
 
 template <int CTRL>
 __device__ __forceinline__ float dpp_f32(float v) {
@@ -120,7 +125,9 @@ struct Im2colBody {
   // neighbouring output columns.  Per input row it needs columns w0-1 .. w0+4:
   // one aligned 16-byte load; the two edge columns are the neighbouring lanes'
   // outer elements, moved with a wavefront-wide DPP shift (lanes 0 and 63 fetch
-  // theirs from memory).  Each of the nine taps is then one 16-byte store.  The
+  // theirs from memory with one single-lane load each; loading them for every
+  // lane from a wave-uniform address instead, as the bilinear kernel does, costs
+  // this kernel 9 %).  Each of the nine taps is then one 16-byte store.  The
   // trip count is wave-uniform so every lane's neighbour is live.
   template <class SB>
   static __device__ __forceinline__ void vec4_3x3(const Args &a, SB &sb) {
@@ -498,15 +505,27 @@ struct UpsampleBilinearBody {
         }
         wl[k] = rn_sub(1.0f, wr[k]);
       }
-      float hl[4][4];  // horizontally interpolated rows 2p-1 .. 2p+2
+      // All loads of the work item are issued before the first use.  Lane 0 has nobody to its left in this
+      // wavefront and lane 63 nobody to its right: their outer columns are loaded from addresses every lane agrees
+      // on (one cache line each, no divergence, nothing to wait for in turn).
+      float2 mm[4];
+      float edge_l[4], edge_r[4];
 #pragma unroll
       for (int r = 0; r < 4; r++) {
         const float *row = pl + (size_t)jr[r] * W1;
-        const float2 m = *reinterpret_cast<const float2 *>(row);
+        mm[r] = *reinterpret_cast<const float2 *>(row);
+        const size_t off = (size_t)(row - a.idata.data);
+        edge_l[r] = a.idata.data[uniform_u64(has_left ? off - 1 : off)];
+        edge_r[r] = a.idata.data[uniform_last_u64(has_right ? off + 2 : off)];
+      }
+      float hl[4][4];  // horizontally interpolated rows 2p-1 .. 2p+2
+#pragma unroll
+      for (int r = 0; r < 4; r++) {
+        const float2 m = mm[r];
         float left = dpp_f32<0x138>(m.y);   // wave_shr:1 -- lane-1's second column
         float right = dpp_f32<0x130>(m.x);  // wave_shl:1 -- lane+1's first column
-        if (lane == 0 && has_left) left = row[-1];
-        if (lane == 63 && has_right) right = row[2];
+        if (lane == 0) left = edge_l[r];
+        if (lane == 63) right = edge_r[r];
         // output 4q: source columns (2q-1, 2q), or (0, 1) with weights (1, 0) at the left edge
         hl[r][0] = rn_add(rn_mul(wl[0], has_left ? left : m.x), rn_mul(wr[0], has_left ? m.x : m.y));
         hl[r][1] = rn_add(rn_mul(wl[1], m.x), rn_mul(wr[1], m.y));

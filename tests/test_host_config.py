@@ -592,13 +592,15 @@ def test_launch_bound_formula_and_built_variants():
         plain.set_barrier_mode(L.HF_BARRIER_BLOCKIDX)
         plain.set_launch_bound(True)
         assert plain.launch_waves[1] == 0                                 # the block-index partition has no bounded build
-    # three more pairs of the shipped list have a second build at the formula's value of their shipped shape --
+    # three more pairs of the shipped list have a second build, at the formula's value of these block shapes --
     # im2col(42, 256) + upsample(22, 512): min(12, 11, 2) = 2 blocks of 768 threads = 6 waves per SIMD;
     # im2col(42, 256) + histogram(19, 640): min(12, 10, 2) = 2 of 896 = 7; im2col + bilinear upsampling (32, 512): 6
     shipped = hfuse_amd.default_config()
-    for k1, k2, w in (("im2col_kernel", "upsample_nearest2d_out_frame", 6), ("im2col_kernel", "kernelHistogram1D", 7),
-                      ("im2col_kernel", "upsample_bilinear2d_out_frame", 6)):
+    for k1, k2, block, w in (("im2col_kernel", "upsample_nearest2d_out_frame", (256, 512), 6),
+                             ("im2col_kernel", "kernelHistogram1D", (256, 640), 7),
+                             ("im2col_kernel", "upsample_bilinear2d_out_frame", (256, 512), 6)):
         p = shipped.plan(shipped.find_fusion(k1, k2), "hfuse_lb")
+        p.set_block(*block)              # whatever shape the list is tuned to today
         assert p.launch_waves == (w, w), (k1, k2, p.launch_waves)
         p.set_launch_waves(8)
         assert p.launch_waves == (w, 8)
