@@ -125,10 +125,11 @@ struct Im2colBody {
   // neighbouring output columns.  Per input row it needs columns w0-1 .. w0+4:
   // one aligned 16-byte load; the two edge columns are the neighbouring lanes'
   // outer elements, moved with a wavefront-wide DPP shift (lanes 0 and 63 fetch
-  // theirs from memory with one single-lane load each; loading them for every
-  // lane from a wave-uniform address instead, as the bilinear kernel does, costs
-  // this kernel 9 %).  Each of the nine taps is then one 16-byte store.  The
-  // trip count is wave-uniform so every lane's neighbour is live.
+  // theirs from memory with one single-lane load each; taking them from a
+  // wave-uniform address instead, as the bilinear kernel does, costs this kernel
+  // 8-9 %: it writes fastest with a slow front end).  Each of the nine taps is
+  // then one 16-byte store.  The trip count is wave-uniform so every lane's
+  // neighbour is live.
   template <class SB>
   static __device__ __forceinline__ void vec4_3x3(const Args &a, SB &sb) {
     const unsigned W = (unsigned)a.width, H = (unsigned)a.height;
