@@ -254,6 +254,22 @@ def test_upsample_bilinear_signed_zeros(cuda):
     assert np.array_equal(out.cpu().numpy().view(np.uint32), want.view(np.uint32))
 
 
+@pytest.mark.parametrize("align", [False, True])
+@pytest.mark.parametrize("offset", [1, 2, 3])
+def test_upsample_bilinear_input_off_the_vector_boundary(cuda, offset, align):
+    """An exact-2x shape whose input starts 4, 8 or 12 bytes past a 16-byte boundary: 8-byte-aligned inputs keep the
+    shifted-lane path, the others take the gathered loads; the bits are the same either way."""
+    n, c, h, w = 2, 3, 10, 12
+    x = uniform((n * c * h * w + offset,), 41 + offset)
+    xd = x.to(cuda)
+    view = xd[offset:].view(n, c, h, w)
+    out = torch.full((n, c, 2 * h, 2 * w), float("nan"), device=cuda)
+    H.launch_native("upsample_bilinear2d_out_frame", H.upsample_bilinear_args(view, out, align))
+    sync()
+    want = O.upsample_bilinear2d(x[offset:].view(n, c, h, w).numpy(), (2 * h, 2 * w), align)
+    assert np.array_equal(out.cpu().numpy().view(np.uint32), want.view(np.uint32))
+
+
 def test_upsample_bilinear_strided_output(cuda):
     x = uniform((2, 3, 6, 6), 17)
     xd = x.to(cuda)
